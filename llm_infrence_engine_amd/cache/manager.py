@@ -26,13 +26,15 @@ from .allocator import NULL_PAGE, OutOfPages, PageAllocator
 
 @dataclass(frozen=True)
 class GroupKey:
-    """What the pages of a group hold (a tuple of ``parts.base.PageTensor``) and for how long."""
+    """What the pages of a group hold (a tuple of ``parts.base.PageTensor``), for how long, and for how many
+    tokens each entry stands (``stride`` > 1: one entry per whole block of that many tokens)."""
 
     tensors: tuple
     window: Optional[int]
+    stride: int = 1
 
-    def values_per_token(self) -> int:
-        return sum(t.heads * t.width for t in self.tensors)
+    def values_per_token(self) -> float:
+        return sum(t.heads * t.width for t in self.tensors) / self.stride
 
 
 @dataclass
@@ -57,36 +59,48 @@ class CacheLayout:
     def __init__(self, run_needs: Sequence[Tuple[object, object, Optional[int]]]):
         self.group_keys: List[GroupKey] = []
         self.group_runs: List[List[int]] = []
-        self.run_group: List[Optional[int]] = []   # group of each run's own or borrowed cache
+        self.run_group: List[Optional[int]] = []   # group of each run's own or borrowed cache (of its first need)
         self.run_entry: List[Optional[int]] = []   # index of the run's pages inside its group
+        self.run_more: List[List[Tuple[int, int]]] = []   # (group, index) of the run's further needs, in their order
         self.run_stores: List[bool] = []
         self.state_runs: List[int] = []
         self.state_needs: Dict[int, object] = {}
+        def as_list(kv):
+            return [] if kv is None else list(kv) if isinstance(kv, (tuple, list)) else [kv]
+
         for i, (kv, state, cache_of) in enumerate(run_needs):
+            needs = as_list(kv)
             if cache_of is not None:
-                if kv is None:
+                if not needs:
                     raise ValueError(f"run {i} reads the cache of run {cache_of} but its mixer keeps no keys and values")
-                src_kv = run_needs[cache_of][0]
-                if src_kv is None or src_kv.tensors != kv.tensors:
+                src = as_list(run_needs[cache_of][0])
+                if len(src) != len(needs) or any(a.tensors != b.tensors or a.stride != b.stride for a, b in zip(src, needs)):
                     raise ValueError(f"run {i} cannot read the cache of run {cache_of}: their pages hold different tensors")
-                if src_kv.window is not None and (kv.window is None or kv.window > src_kv.window):
-                    raise ValueError(f"run {i} looks further back than run {cache_of}, whose cache it reads, keeps keys")
+                for a, b in zip(src, needs):
+                    if a.window is not None and (b.window is None or b.window > a.window):
+                        raise ValueError(f"run {i} looks further back than run {cache_of}, whose cache it reads, keeps keys")
                 self.run_group.append(self.run_group[cache_of])
                 self.run_entry.append(self.run_entry[cache_of])
+                self.run_more.append(list(self.run_more[cache_of]))
                 self.run_stores.append(False)
-            elif kv is not None:
-                key = GroupKey(tuple(kv.tensors), kv.window)
-                if key not in self.group_keys:
-                    self.group_keys.append(key)
-                    self.group_runs.append([])
-                g = self.group_keys.index(key)
-                self.run_group.append(g)
-                self.run_entry.append(len(self.group_runs[g]))
-                self.group_runs[g].append(i)
+            elif needs:
+                placed = []
+                for need in needs:
+                    key = GroupKey(tuple(need.tensors), need.window, need.stride)
+                    if key not in self.group_keys:
+                        self.group_keys.append(key)
+                        self.group_runs.append([])
+                    g = self.group_keys.index(key)
+                    placed.append((g, len(self.group_runs[g])))
+                    self.group_runs[g].append(i)
+                self.run_group.append(placed[0][0])
+                self.run_entry.append(placed[0][1])
+                self.run_more.append(placed[1:])
                 self.run_stores.append(True)
             else:
                 self.run_group.append(None)
                 self.run_entry.append(None)
+                self.run_more.append([])
                 self.run_stores.append(False)
             if state is not None:
                 self.state_runs.append(i)
@@ -96,8 +110,8 @@ class CacheLayout:
     def bytes_per_token(self, bytes_per_value: int) -> int:
         """Stored bytes per token over all runs that keep a cache (for keys and values: layers x 2 x kv heads
         x head size x bytes, src/miniserve/cache.py:27-29)."""
-        return sum(len(runs) * key.values_per_token() * bytes_per_value
-                   for key, runs in zip(self.group_keys, self.group_runs))
+        return int(-(-sum(len(runs) * key.values_per_token() * bytes_per_value
+                          for key, runs in zip(self.group_keys, self.group_runs)) // 1))
 
 
 class CacheManager:
@@ -174,11 +188,14 @@ class CacheManager:
         for k, p in enumerate(pages):
             changed[base + k] = int(p)
 
+    def entries(self, gi: int, n_tokens: int) -> int:
+        """Entries a request of ``n_tokens`` tokens holds in group ``gi``: one per token, or one per whole block."""
+        return n_tokens // self.groups[gi].key.stride
+
     def pages_to_grow(self, req_id, new_len: int) -> List[int]:
         """Pages each group must hand out so that the request can hold ``new_len`` tokens."""
         h = self._held[req_id]
-        need = -(-new_len // self.page_size)
-        return [max(0, need - h.next_page[i]) for i in range(len(self.groups))]
+        return [max(0, -(-self.entries(i, new_len) // self.page_size) - h.next_page[i]) for i in range(len(self.groups))]
 
     def can_grow(self, req_id, new_len: int, reserve: int = 0) -> bool:
         """True if every group has the pages for ``new_len`` tokens and ``reserve`` more."""
@@ -192,7 +209,8 @@ class CacheManager:
         h = self._held[req_id]
         fit = self.max_len - h.computed
         for i, g in enumerate(self.groups):
-            room = (h.next_page[i] + max(0, g.allocator.num_free() - reserve)) * self.page_size - h.computed
+            s = g.key.stride     # pages for e entries hold the tokens up to the one before entry e + 1 would be due
+            room = (h.next_page[i] + max(0, g.allocator.num_free() - reserve)) * self.page_size * s + (s - 1) - h.computed
             fit = min(fit, room)
         return fit
 
@@ -216,7 +234,7 @@ class CacheManager:
         h = self._held[req_id]
         if computed < h.computed:
             raise ValueError("a request's stored tokens cannot shrink; free it and add it again")
-        if self.groups and computed > min(h.next_page) * self.page_size:
+        if any(self.entries(i, computed) > h.next_page[i] * self.page_size for i in range(len(self.groups))):
             raise ValueError(f"request {req_id!r}: {computed} tokens stored but pages for fewer were allocated")
         h.computed = computed
         for i, g in enumerate(self.groups):

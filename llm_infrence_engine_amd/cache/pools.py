@@ -60,10 +60,20 @@ class CachePools:
 
     def kv_view(self, run: int, table_rows: torch.Tensor, slot_mapping: torch.Tensor) -> KVView:
         """The run's pages with its group's table; ``table_rows`` [R]: the rows of the step's requests."""
-        g, e = self.layout.run_group[run], self.layout.run_entry[run]
+        return self._view(run, self.layout.run_group[run], self.layout.run_entry[run], table_rows, slot_mapping, ())
+
+    def _view(self, run, g, e, table_rows, slot_mapping, more) -> KVView:
+        key = self.layout.group_keys[g]
         return KVView({name: t[e] for name, t in self.pages[g].items()}, dict(self.transposed[g]), self.tables[g],
-                      slot_mapping, store=self.layout.run_stores[run], window=self.layout.group_keys[g].window,
-                      table_rows=table_rows)
+                      slot_mapping, store=self.layout.run_stores[run], window=key.window, table_rows=table_rows,
+                      stride=key.stride, more=tuple(more))
+
+    def kv_views(self, run: int, table_rows: torch.Tensor, slots) -> KVView:
+        """As ``kv_view`` with the step's slots of every group (``slots[g]``): the view of the run's first need, the
+        views of its further needs in ``more``."""
+        more = [self._view(run, g, e, table_rows, slots[g], ()) for g, e in self.layout.run_more[run]]
+        g = self.layout.run_group[run]
+        return self._view(run, g, self.layout.run_entry[run], table_rows, slots[g], more)
 
     def apply_updates(self, index: Sequence[torch.Tensor], value: Sequence[torch.Tensor], counts: torch.Tensor,
                       max_updates: int) -> None:

@@ -25,7 +25,7 @@ int ms_bias_add(void* x, const float* bias, int n_rows, int width, int dtype, hi
 int ms_max_cache_groups();
 int ms_decode_advance(const int* prev_tokens, int* token_ids, int* positions, int* context_lens, const int* n_live,
                       const int* table_rows, int* draw_index, const int* const* tables, int* const* slots,
-                      int n_groups, int table_stride, int page_size, int n_rows, hipStream_t stream);
+                      const int* strides, int n_groups, int table_stride, int page_size, int n_rows, hipStream_t stream);
 
 // Block tables kept on the device: tables[g][index[g][i]] = value[g][i] for i < counts[g] (counts: device ints),
 // every index at most once per group; max_updates bounds counts, table_elems bounds the indices.
@@ -231,9 +231,10 @@ int ms_selective_scan(const void* x, long long x_stride, const float* dt_in, con
 
 // ---- routed experts (csrc/experts.hip)
 int ms_gelu(const void* x, void* out, long long total, int dtype, hipStream_t stream);
-// softmax over logits[n, :n_out] (rows ld apart), the `top` largest of score + correction: ids / weights [n, top]
+// softmax over logits[n, :n_out] (rows ld apart; sigmoid_scores: each logit's own sigmoid instead), the `top` largest of
+// score + correction: ids / weights [n, top]
 int ms_moe_route(const float* logits, long long ld, const float* correction, int n_tokens, int n_out, int top, int* ids,
-                 float* weights, hipStream_t stream);
+                 float* weights, int sigmoid_scores, hipStream_t stream);
 int ms_moe_tile_rows();
 int ms_moe_wide_tile_rows();
 // rows [tiles * tile] and tile_expert [tiles] from ids [n_items]; ids >= n_experts take no row; tile: ms_moe_tile_rows()
@@ -255,6 +256,36 @@ int ms_grouped_gemm(const void* in, long long in_stride, const void* w, const in
                     int dtype, int out_dtype, hipStream_t stream);
 int ms_moe_combine(const float* part, const int* ids, const float* weights, const void* h, long long h_stride,
                    const void* shared, int shared_dtype, const float* gate, long long gate_stride, float* out,
-                   int n_tokens, int top, int n_experts, int hidden, int dtype, hipStream_t stream);
+                   int n_tokens, int top, int n_experts, int hidden, int dtype, hipStream_t stream);   // weights null: all 1
+
+// ---- layer norm and the token's side input (csrc/layer_norm.hip)
+int ms_layer_norm(float* x, const void* delta, int delta_dtype, const float* dscale, const float* w, const int* rows,
+                  void* out, int n_rows, int H, float eps, int write_back, int out_dtype, hipStream_t stream);
+int ms_token_side(float* x, const void* delta, int delta_dtype, const float* dscale, const int* token_ids, const void* table,
+                  long long table_stride, int part, const void* G, const void* P, const float* w, int n_tokens, int H, int d,
+                  float eps, int dtype, hipStream_t stream);
+// ---- minGRU (csrc/mingru.hip)
+int ms_mingru_scan(const void* zxg, long long in_stride, const float* bz, const float* bx, float* state, const int* q_start,
+                   const int* state_slots, void* out, long long out_stride, int n_requests, int C, int long_portions,
+                   int dtype, hipStream_t stream);
+// ---- window + pooled blocks attention (csrc/pooled_attention.hip)
+int ms_pairs_rotate_store(void* qkv, long long stride, const int* positions, const float* inv_freq, const float* inv_freq_v,
+                          const int* slots, void* k_pages, void* v_pages, int n_tokens, int num_heads, int num_kv_heads,
+                          int head_dim, int value_dim, int rot_dims, int page_size, int dtype, hipStream_t stream);
+int ms_pool_store(const void* k_pages, const void* v_pages, const int* table, int table_stride, const int* table_rows,
+                  const int* token_req, const int* positions, const int* pool_slots, void* pk_pages, void* pv_pages,
+                  int n_tokens, int num_kv_heads, int head_dim, int value_dim, int page_size, int pool, int dtype,
+                  hipStream_t stream);
+int ms_pooled_attention(const void* q, long long q_stride, const void* k_pages, const void* v_pages, const int* table,
+                        const void* pk_pages, const void* pv_pages, const int* pool_table, int table_stride,
+                        const int* table_rows, const int* n_live_tokens, const int* token_req, const int* positions,
+                        const float* inv_freq_v, void* out, long long out_stride, int n_tokens, int num_heads,
+                        int num_kv_heads, int head_dim, int value_dim, int page_size, float scale, int size, int pool,
+                        int dtype, hipStream_t stream);
+// ---- gated activations (csrc/glu.hip)
+int ms_clamped_glu(const void* gu, long long in_stride, void* out, long long out_stride, int n_rows, int F, float limit,
+                   float alpha, int dtype, hipStream_t stream);
+int ms_scaled_swiglu(const void* gu, long long in_stride, const float* factor, const int* row_item, void* out,
+                     long long out_stride, int n_rows, int F, int dtype, hipStream_t stream);
 
 }  // extern "C"

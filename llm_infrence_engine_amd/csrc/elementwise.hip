@@ -509,6 +509,7 @@ struct AdvanceArgs {
   int* draw_index;
   const int* tables[MS_MAX_GROUPS];
   int* slots[MS_MAX_GROUPS];
+  int strides[MS_MAX_GROUPS];
   int n_groups, table_stride, page_size, n_rows;
 };
 
@@ -521,23 +522,30 @@ __global__ void decode_advance_kernel(AdvanceArgs a) {
   a.token_ids[r] = a.prev_tokens[r];
   if (a.draw_index) a.draw_index[r] += 1;     // the next draw of a request that samples is its next
   const size_t row = a.table_rows ? a.table_rows[r] : r;
-  for (int g = 0; g < a.n_groups; ++g)
-    a.slots[g][r] = a.tables[g][row * a.table_stride + pos / a.page_size] * a.page_size + pos % a.page_size;
+  for (int g = 0; g < a.n_groups; ++g) {
+    const int s = a.strides[g];       // tokens per entry: a group with s > 1 stores with a block's last token only
+    const int e = (pos + 1) / s - 1;
+    a.slots[g][r] = (pos + 1) % s ? -1 : a.tables[g][row * a.table_stride + e / a.page_size] * a.page_size + e % a.page_size;
+  }
 }
 
 extern "C" int ms_max_cache_groups() { return MS_MAX_GROUPS; }
 
 extern "C" int ms_decode_advance(const int* prev_tokens, int* token_ids, int* positions, int* context_lens,
                                  const int* n_live, const int* table_rows, int* draw_index,
-                                 const int* const* tables, int* const* slots, int n_groups, int table_stride,
-                                 int page_size, int n_rows, hipStream_t stream) {
+                                 const int* const* tables, int* const* slots, const int* strides, int n_groups,
+                                 int table_stride, int page_size, int n_rows, hipStream_t stream) {
   if (n_rows <= 0) return MS_OK;
   if (n_groups < 0 || n_groups > MS_MAX_GROUPS || table_stride <= 0 || page_size <= 0) return MS_BAD_ARG;
   AdvanceArgs a;
   a.prev_tokens = prev_tokens; a.token_ids = token_ids; a.positions = positions; a.context_lens = context_lens;
   a.n_live = n_live; a.table_rows = table_rows; a.draw_index = draw_index; a.n_groups = n_groups; a.table_stride = table_stride;
   a.page_size = page_size; a.n_rows = n_rows;
-  for (int g = 0; g < MS_MAX_GROUPS; ++g) { a.tables[g] = g < n_groups ? tables[g] : nullptr; a.slots[g] = g < n_groups ? slots[g] : nullptr; }
+  for (int g = 0; g < MS_MAX_GROUPS; ++g) {
+    a.tables[g] = g < n_groups ? tables[g] : nullptr;
+    a.slots[g] = g < n_groups ? slots[g] : nullptr;
+    a.strides[g] = g < n_groups && strides && strides[g] > 0 ? strides[g] : 1;
+  }
   decode_advance_kernel<<<dim3((n_rows + 63) / 64), dim3(64), 0, stream>>>(a);
   return ms_launch_status();
 }

@@ -31,10 +31,11 @@ __global__ void gelu_kernel(const T* __restrict__ x, T* __restrict__ out, size_t
     out[i] = from_float<T>(gelu_erf(to_float(x[i])));
 }
 
-// One wave per token.  Ties go to the lower index.
+// One wave per token.  Ties go to the lower index.  sigmoid_scores: every score is the sigmoid of its own logit
+// instead of the softmax over all of them.
 __global__ void __launch_bounds__(256)
 moe_route_kernel(const float* __restrict__ logits, size_t ld, const float* __restrict__ correction, int n_tokens,
-                 int n_out, int top, int* __restrict__ ids, float* __restrict__ weights) {
+                 int n_out, int top, int* __restrict__ ids, float* __restrict__ weights, int sigmoid_scores) {
   const int lane = threadIdx.x & (MS_WAVE - 1);
   const int n = blockIdx.x * (blockDim.x / MS_WAVE) + threadIdx.x / MS_WAVE;
   if (n >= n_tokens) return;
@@ -52,11 +53,11 @@ moe_route_kernel(const float* __restrict__ logits, size_t ld, const float* __res
 #pragma unroll
   for (int i = 0; i < ROUTE_MAX_PER_LANE; ++i) {
     const int e = lane + i * MS_WAVE;
-    s[i] = e < n_out ? expf(s[i] - big) : 0.f;
+    s[i] = e < n_out ? (sigmoid_scores ? 1.0f / (1.0f + expf(-s[i])) : expf(s[i] - big)) : 0.f;
     sum += s[i];
   }
   sum = wave_sum(sum);
-  const float inv = 1.0f / sum;
+  const float inv = sigmoid_scores ? 1.0f : 1.0f / sum;
 #pragma unroll
   for (int i = 0; i < ROUTE_MAX_PER_LANE; ++i) {
     const int e = lane + i * MS_WAVE;
@@ -377,7 +378,7 @@ moe_combine_kernel(const float* __restrict__ part, const int* __restrict__ ids, 
   __shared__ float s_w[ROUTE_MAX_TOP];
   if ((int)threadIdx.x < top) {
     s_id[threadIdx.x] = ids[(size_t)n * top + threadIdx.x];
-    s_w[threadIdx.x] = weights[(size_t)n * top + threadIdx.x];
+    s_w[threadIdx.x] = weights ? weights[(size_t)n * top + threadIdx.x] : 1.0f;
   }
   __syncthreads();
   float g = 0.f;
@@ -406,12 +407,12 @@ extern "C" int ms_gelu(const void* x, void* out, long long total, int dtype, hip
 }
 
 extern "C" int ms_moe_route(const float* logits, long long ld, const float* correction, int n_tokens, int n_out, int top,
-                            int* ids, float* weights, hipStream_t stream) {
+                            int* ids, float* weights, int sigmoid_scores, hipStream_t stream) {
   if (n_tokens <= 0) return MS_OK;
   if (n_out <= 0 || top <= 0 || top > n_out) return MS_BAD_ARG;
   if (n_out > ROUTE_MAX_PER_LANE * MS_WAVE || top > ROUTE_MAX_TOP) return MS_UNSUPPORTED;
   moe_route_kernel<<<(n_tokens + 3) / 4, 256, 0, stream>>>(logits, (size_t)ld, correction, n_tokens, n_out, top, ids,
-                                                           weights);
+                                                           weights, sigmoid_scores);
   return ms_launch_status();
 }
 

@@ -175,12 +175,17 @@ class BatchBuilder:
                 wanted.append(int(q_start[r]) + int(w))
         slots = []
         token_rows = rows[token_req]
-        last_page = (ctx_lens + steps - 2) // ps
         for g in m.groups:
-            page = g.tables[token_rows, positions // ps]
-            if (page == 0).any() or (g.tables[rows, last_page] == 0).any():
+            s = g.key.stride
+            # a group that keeps one entry per block of s tokens stores it with the block's last token
+            stores = (positions + 1) % s == 0
+            entry = (positions + 1) // s - 1
+            page = np.where(stores, g.tables[token_rows, np.maximum(entry, 0) // ps], 1)
+            held = (ctx_lens + steps - 1) // s            # entries each request holds after the last of the steps
+            last = g.tables[rows, np.maximum(held - 1, 0) // ps]
+            if (page == 0).any() or ((held > 0) & (last == 0)).any():
                 raise RuntimeError("a token of this step has no page; grow the request before building the batch")
-            slots.append(page.astype(np.int32) * ps + positions % ps)
+            slots.append(np.where(stores, page.astype(np.int32) * ps + entry % ps, -1).astype(np.int32))
         return _Described(N, R, token_ids.astype(np.int32), positions, token_req, slots, q_start, ctx_lens, rows,
                           rows[starts == 0], np.asarray(wanted, dtype=np.int32), q_lens, starts)
 

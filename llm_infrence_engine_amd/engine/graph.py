@@ -52,7 +52,8 @@ def portion_graph_limit(model) -> int:
     15 us each), at a rate of matrix work that short portions reach.  Beyond that the host hides behind the
     GPU anyway and a graph's padding up to its bucket would only add work."""
     weights = sum(s.shape[0] * s.shape[1] for s in model.tensor_specs() if s.role == "matrix" and len(s.shape) == 2)
-    ends = sum(s.shape[0] * s.shape[1] for part in (model.embedding, model.head) for s in part.tensor_specs())
+    ends = sum(s.shape[0] * s.shape[1] for part in (model.embedding, model.head) for s in part.tensor_specs()
+               if s.role == "matrix" and len(s.shape) == 2)
     per_token = 2.0 * max(1, weights - ends)
     launches = 9 * len(model.spec.order)
     tokens = launches * 13e-6 * 0.4e15 / per_token
@@ -188,7 +189,8 @@ class StepGraphs:
                 if k > 0:      # n_live is 0 in the buffer while capturing and warming up: nothing moves
                     ops.decode_advance(bk.tokens[k - 1], f["token_ids"], f["positions"], f["context_lens"], f["n_live"],
                                        f["state_slots"], runner.pools.tables, bk.slots, self.manager.page_size,
-                                       f["draw_index"] if bk.sampled else None)
+                                       f["draw_index"] if bk.sampled else None,
+                                       strides=[g.key.stride for g in self.manager.groups])
                     ctx.shared.clear()
                 bk.logits = model.head_logits(*model.forward_hidden(ctx, caches), ctx.logit_rows)
                 if bk.sampled:     # rows without a temperature (padding rows too) take the first maximum

@@ -31,6 +31,10 @@ class ModelRunner:
         if len(self.layout.group_keys) > ops.MAX_CACHE_GROUPS:
             raise ValueError(f"the model's runs fall into {len(self.layout.group_keys)} cache groups; the kernels that "
                              f"keep block tables and slots serve at most {ops.MAX_CACHE_GROUPS}")
+        if isinstance(num_pages, int):
+            # a group that keeps one entry per block of tokens needs that much less (and a page in part per request)
+            num_pages = [num_pages if key.stride == 1 else -(-num_pages // key.stride) + max_requests
+                         for key in self.layout.group_keys]
         self.manager = CacheManager(self.layout, page_size, num_pages, max_requests, max_len)
         self.pools = CachePools(self.layout, page_size, num_pages, max_requests, self.rt,
                                 self.manager.max_pages_per_request)
@@ -57,7 +61,7 @@ class ModelRunner:
         out = []
         for i in range(len(self.model.spec.order)):
             g = self.layout.run_group[i]
-            kv = self.pools.kv_view(i, table_rows, slots[g]) if g is not None else None
+            kv = self.pools.kv_views(i, table_rows, slots) if g is not None else None
             state = self.pools.state_view(i) if i in self.layout.state_needs else None
             out.append(RunCache(kv, state))
         return out

@@ -28,7 +28,7 @@ _SIGNATURES = {
                             _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_qkv_rope_store": [_c_ptr, _c_ll, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                           _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
-    "ms_decode_advance": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
+    "ms_decode_advance": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
                           _c_int, _c_ptr],
     "ms_max_cache_groups": [],
     "ms_table_update": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ll, _c_ptr],
@@ -100,7 +100,21 @@ _SIGNATURES = {
     "ms_selective_scan": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_ptr,
                           _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_gelu": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
-    "ms_moe_route": [_c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
+    "ms_moe_route": [_c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
+    "ms_layer_norm": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
+    "ms_token_side": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+                      _c_int, _c_float, _c_int, _c_ptr],
+    "ms_mingru_scan": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int,
+                       _c_ptr],
+    "ms_pairs_rotate_store": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
+                              _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_pool_store": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
+                      _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_pooled_attention": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                            _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
+                            _c_int, _c_int, _c_ptr],
+    "ms_clamped_glu": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_int, _c_int, _c_float, _c_float, _c_int, _c_ptr],
+    "ms_scaled_swiglu": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_ptr],
     "ms_moe_tile_rows": [],
     "ms_moe_wide_tile_rows": [],
     "ms_gemm_tiled_grouped_rows": [],
@@ -281,10 +295,12 @@ def _pointer_array(tensors):
 
 def decode_advance(prev_tokens: torch.Tensor, token_ids: torch.Tensor, positions: torch.Tensor,
                    context_lens: torch.Tensor, n_live: torch.Tensor, table_rows: Optional[torch.Tensor], tables, slots,
-                   page_size: int, draw_index: Optional[torch.Tensor] = None) -> None:
+                   page_size: int, draw_index: Optional[torch.Tensor] = None, strides=None) -> None:
     """Between two decode steps queued back to back: rows below ``n_live[0]`` move one position on, take
     ``prev_tokens`` as their input, count ``draw_index`` up by one and get their new slots from ``tables`` (one
-    [table rows, width] per cache group; row r of the batch has the table row ``table_rows[r]``, or r without it)."""
+    [table rows, width] per cache group; row r of the batch has the table row ``table_rows[r]``, or r without it).
+    ``strides``: per group the tokens an entry stands for (1, the default: an entry per token; s > 1: the group stores with
+    the last token of a block of s, other tokens get the slot -1)."""
     R = token_ids.numel()
     for t, name in ((prev_tokens, "prev_tokens"), (token_ids, "token_ids"), (positions, "positions"),
                     (context_lens, "context_lens")):
@@ -302,8 +318,10 @@ def decode_advance(prev_tokens: torch.Tensor, token_ids: torch.Tensor, positions
         _check(sl, "slots", torch.int32, (R,))
     keep_t, tp = _pointer_array(tables)
     keep_s, sp = _pointer_array(slots)
+    st = (ctypes.c_int * max(1, len(tables)))(*[int(v) for v in (strides or [1] * len(tables))])
     _call("ms_decode_advance", prev_tokens.data_ptr(), token_ids.data_ptr(), positions.data_ptr(),
-          context_lens.data_ptr(), n_live.data_ptr(), _ptr(table_rows), _ptr(draw_index), tp, sp, len(tables), width,
+          context_lens.data_ptr(), n_live.data_ptr(), _ptr(table_rows), _ptr(draw_index), tp, sp,
+          ctypes.cast(st, ctypes.c_void_p), len(tables), width,
           page_size, R, _stream())
 
 
@@ -1244,9 +1262,13 @@ def gelu(x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, n_out: Optional[int] = None):
-    """Scores = softmax(logits[:, :n_out]); the ``top`` largest of scores + correction are chosen (the lower index on a
-    tie).  Returns (ids int32 [N, top], their scores float [N, top]).  logits float [N, >= n_out]."""
+def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, n_out: Optional[int] = None,
+              scores: str = "softmax"):
+    """Scores = softmax(logits[:, :n_out]) (``scores`` "sigmoid": every logit's own sigmoid); the ``top`` largest of
+    scores + correction are chosen (the lower index on a tie).  Returns (ids int32 [N, top], their scores float [N, top]).
+    logits float [N, >= n_out]."""
+    if scores not in ("softmax", "sigmoid"):
+        raise ValueError(f"router scores are 'softmax' or 'sigmoid', not {scores!r}")
     ld = _rows2d(logits, "logits", torch.float32)
     N = logits.shape[0]
     n_out = logits.shape[1] if n_out is None else n_out
@@ -1256,7 +1278,8 @@ def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int
         _check(correction, "correction", torch.float32, (n_out,))
     ids = torch.empty((N, top), dtype=torch.int32, device=logits.device)
     weights = torch.empty((N, top), dtype=torch.float32, device=logits.device)
-    _call("ms_moe_route", logits.data_ptr(), ld, _ptr(correction), N, n_out, top, ids.data_ptr(), weights.data_ptr(), _stream())
+    _call("ms_moe_route", logits.data_ptr(), ld, _ptr(correction), N, n_out, top, ids.data_ptr(), weights.data_ptr(),
+          int(scores == "sigmoid"), _stream())
     return ids, weights
 
 
@@ -1344,7 +1367,8 @@ def moe_combine(part: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, h:
     is fine); out float [N, H]."""
     N, top = ids.shape
     _check(ids, "ids", torch.int32)
-    _check(weights, "weights", torch.float32, (N, top))
+    if weights is not None:      # None: every choice weighs 1
+        _check(weights, "weights", torch.float32, (N, top))
     H = out.shape[1]
     _check(part, "part", torch.float32, (N * top, H))
     hs = _rows2d(h, "h", None, H)
@@ -1357,6 +1381,213 @@ def moe_combine(part: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, h:
         if gate.dim() != 1 or gate.shape[0] != N:
             raise ValueError("gate must be one float per token")
         gs = gate.stride(0) if N > 1 else 1
-    _call("ms_moe_combine", part.data_ptr(), ids.data_ptr(), weights.data_ptr(), h.data_ptr(), hs, _ptr(shared), scode,
+    _call("ms_moe_combine", part.data_ptr(), ids.data_ptr(), _ptr(weights), h.data_ptr(), hs, _ptr(shared), scode,
           _ptr(gate), gs, out.data_ptr(), N, top, n_experts, H, _code(h.dtype), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ layer norm, side input
+def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out: Optional[torch.Tensor],
+               delta: Optional[torch.Tensor] = None, delta_scale: Optional[torch.Tensor] = None,
+               rows: Optional[torch.Tensor] = None, write_back: bool = True):
+    """out[r] = weight * (v - mean v) / sqrt(mean (v - mean v)^2 + eps) with v = x[rows[r]] (+ delta_scale o delta[rows[r]]).
+    x float32 [N, H] is the residual stream; with ``delta`` [N, H] the sum is written back to x (unless ``write_back`` is
+    False).  ``weight`` None: only the sum.  ``out`` may be x itself (float): the rows are normed in place."""
+    _check(x, "x", torch.float32)
+    N, H = x.shape
+    n_rows = N
+    if rows is not None:
+        _check(rows, "rows", torch.int32)
+        n_rows = rows.numel()
+    if weight is not None:
+        _check(weight, "weight", torch.float32, (H,))
+        _check(out, "out", None, (n_rows, H))
+    dcode = 0
+    if delta is not None:
+        _check(delta, "delta", None, (N, H))
+        dcode = _code(delta.dtype)
+        if delta_scale is not None:
+            _check(delta_scale, "delta_scale", torch.float32, (H,))
+    elif delta_scale is not None:
+        raise ValueError("a scale without an addend")
+    _call("ms_layer_norm", x.data_ptr(), _ptr(delta), dcode, _ptr(delta_scale), _ptr(weight), _ptr(rows),
+          _ptr(out) if weight is not None else None, n_rows, H, float(eps), int(write_back),
+          _code(out.dtype) if weight is not None else F32, _stream())
+    return out
+
+
+def token_side(x: torch.Tensor, token_ids: torch.Tensor, table: torch.Tensor, part: int, gate: torch.Tensor,
+               proj: torch.Tensor, weight: torch.Tensor, eps: float, delta: Optional[torch.Tensor] = None,
+               delta_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x[n] <- v + y / sqrt(mean y^2 + eps) o weight, with v = x[n] (+ delta_scale o delta[n]), c = table[token_ids[n],
+    part d : (part + 1) d], y = proj (gelu_tanh(gate v) o c).  x float32 [N, H]; table [V, parts d]; gate [d, H]; proj
+    [H, d]; weight float [H]."""
+    _check(x, "x", torch.float32)
+    N, H = x.shape
+    d = gate.shape[0]
+    _check(gate, "gate", table.dtype, (d, H))
+    _check(proj, "proj", table.dtype, (H, d))
+    _check(table, "table")
+    if table.dim() != 2 or (part + 1) * d > table.shape[1] or part < 0:
+        raise ValueError(f"part {part} of {d} entries is not within the table's rows of {table.shape[1]}")
+    _check(token_ids, "token_ids", torch.int32, (N,))
+    _check(weight, "weight", torch.float32, (H,))
+    dcode = 0
+    if delta is not None:
+        _check(delta, "delta", None, (N, H))
+        dcode = _code(delta.dtype)
+        if delta_scale is not None:
+            _check(delta_scale, "delta_scale", torch.float32, (H,))
+    _call("ms_token_side", x.data_ptr(), _ptr(delta), dcode, _ptr(delta_scale), token_ids.data_ptr(), table.data_ptr(),
+          table.shape[1], int(part), gate.data_ptr(), proj.data_ptr(), weight.data_ptr(), N, H, d, float(eps),
+          _code(table.dtype), _stream())
+    return x
+
+
+# ------------------------------------------------------------------------------------------------ minGRU
+def mingru_scan(zxg: torch.Tensor, bias_z: Optional[torch.Tensor], bias_x: Optional[torch.Tensor], state: torch.Tensor,
+                ctx, out: torch.Tensor) -> torch.Tensor:
+    """The minGRU recurrence over the step's portions, from and into ``state`` float [slots, C]: with the thirds pz | px | pg
+    of a row of zxg [N, 3C]: z = sigmoid(pz + bias_z); u = px + bias_x; c = u + 1/2 (u >= 0) or sigmoid(u);
+    S <- (1 - z) S + z c; out = S * silu(pg)."""
+    C = state.shape[1]
+    stride = _rows2d(zxg, "zxg", None, 3 * C)
+    N = zxg.shape[0]
+    os_ = _rows2d(out, "out", zxg.dtype, C)
+    if out.shape[0] != N:
+        raise ValueError("out has one row per token")
+    for b, name in ((bias_z, "bias_z"), (bias_x, "bias_x")):
+        if b is not None:
+            _check(b, name, torch.float32, (C,))
+    _check(state, "state", torch.float32, (None, C))
+    R = ctx.num_requests
+    _check(ctx.q_start, "q_start", torch.int32, (R + 1,))
+    _check(ctx.state_slots, "state_slots", torch.int32, (R,))
+    _call("ms_mingru_scan", zxg.data_ptr(), stride, _ptr(bias_z), _ptr(bias_x), state.data_ptr(), ctx.q_start.data_ptr(),
+          ctx.state_slots.data_ptr(), out.data_ptr(), os_, R, C, int(ctx.max_q_len > 8), _code(zxg.dtype), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ window + pooled blocks
+def _token_pages(kv, names=("k", "v")):
+    k, v = kv.pages[names[0]], kv.pages[names[1]]
+    if kv.transposed.get(names[0]) or kv.transposed.get(names[1]):
+        raise ValueError("these kernels read pages as [page, head, slot, width]")
+    _check(k, "k pages")
+    _check(v, "v pages", k.dtype, (k.shape[0], k.shape[1], k.shape[2], None))
+    return k, v
+
+
+def pairs_rotate_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
+                       rot_dims: int, positions: torch.Tensor, inv_freq: torch.Tensor, inv_freq_v: torch.Tensor,
+                       kv) -> torch.Tensor:
+    """Rows of the packed projection [N, nh d + nkv d + nkv dv]: q and k heads turn over their first ``rot_dims`` entries
+    (entries 2m, 2m + 1 by positions[n] * inv_freq[m]), value heads over all their entries (by positions[n] *
+    inv_freq_v[m]); q in place, k and v into ``kv``'s pages at the tokens' slots (``kv`` None or not storing: q only)."""
+    N = qkv.shape[0]
+    width = (num_heads + num_kv_heads) * head_dim + num_kv_heads * value_dim
+    stride = _rows2d(qkv, "qkv", None, width)
+    _check(positions, "positions", torch.int32, (N,))
+    _check(inv_freq, "inv_freq", torch.float32, (rot_dims // 2,))
+    _check(inv_freq_v, "inv_freq_v", torch.float32, (value_dim // 2,))
+    store = kv is not None and kv.store
+    k = v = None
+    page_size = 1
+    if store:
+        k, v = _token_pages(kv)
+        _check(k, "k pages", qkv.dtype, (None, num_kv_heads, None, head_dim))
+        _check(v, "v pages", qkv.dtype, (None, num_kv_heads, None, value_dim))
+        _check(kv.slot_mapping, "slot_mapping", torch.int32, (N,))
+        page_size = k.shape[2]
+    _call("ms_pairs_rotate_store", qkv.data_ptr(), stride, positions.data_ptr(), inv_freq.data_ptr(), inv_freq_v.data_ptr(),
+          kv.slot_mapping.data_ptr() if store else None, _ptr(k), _ptr(v), N, num_heads, num_kv_heads, head_dim, value_dim,
+          rot_dims, page_size, _code(qkv.dtype), _stream())
+    return qkv
+
+
+def pool_store(kv, pooled, ctx, pool: int) -> None:
+    """For every token of the step that ends a block of ``pool`` tokens (its slot in ``pooled`` is not negative): the means
+    of the block's keys and values, read back from ``kv``'s pages, go into ``pooled``'s pages "k" and "v"."""
+    k, v = _token_pages(kv)
+    pk, pv = _token_pages(pooled)
+    P, nkv, page_size, d = k.shape
+    dv = v.shape[3]
+    _check(pk, "pooled k", k.dtype, (None, nkv, page_size, d))
+    _check(pv, "pooled v", k.dtype, (None, nkv, page_size, dv))
+    N = ctx.num_tokens
+    _check(pooled.slot_mapping, "pooled slots", torch.int32, (N,))
+    _check(kv.block_table, "block_table", torch.int32)
+    _call("ms_pool_store", k.data_ptr(), v.data_ptr(), kv.block_table.data_ptr(), kv.block_table.shape[1],
+          _ptr(kv.table_rows), ctx.token_req.data_ptr(), ctx.positions.data_ptr(), pooled.slot_mapping.data_ptr(),
+          pk.data_ptr(), pv.data_ptr(), N, nkv, d, dv, page_size, int(pool), _code(k.dtype), _stream())
+
+
+def pooled_attention(q: torch.Tensor, kv, pooled, ctx, out: torch.Tensor, num_heads: int, scale: float, size: int,
+                     pool: int, inv_freq_v: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[n, h] = softmax over the last ``size`` tokens up to n's position and over the pooled entry of every block of
+    ``pool`` tokens that lies wholly before that window (block b: b pool + pool - 1 <= position - size), one softmax for
+    both; tokens from ``kv``'s pages, block b from entry b of ``pooled``'s (None: no blocks).  With ``inv_freq_v`` the
+    output's entries 2m, 2m + 1 are turned by -position * inv_freq_v[m].  q [N, >= nh d] row slices; out [N, nh dv]."""
+    k, v = _token_pages(kv)
+    P, nkv, page_size, d = k.shape
+    dv = v.shape[3]
+    _check(q, "q", k.dtype, contiguous=False)
+    N = q.shape[0]
+    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < num_heads * d:
+        raise ValueError(f"q must be [N, >= {num_heads * d}] with unit stride along rows, got {list(q.shape)}")
+    _check(out, "out", k.dtype, (N, num_heads * dv))
+    if num_heads % nkv:
+        raise ValueError(f"{num_heads} query heads cannot share {nkv} key/value heads")
+    pk = pv = ptab = None
+    if pooled is not None and pool > 0:
+        pk, pv = _token_pages(pooled)
+        _check(pk, "pooled k", k.dtype, (None, nkv, page_size, d))
+        _check(pv, "pooled v", k.dtype, (None, nkv, page_size, dv))
+        ptab = pooled.block_table
+        _check(ptab, "pooled table", torch.int32, tuple(kv.block_table.shape))
+    else:
+        pool = 0
+    if inv_freq_v is not None:
+        _check(inv_freq_v, "inv_freq_v", torch.float32, (dv // 2,))
+    _check(ctx.token_req, "token_req", torch.int32, (N,))
+    _check(ctx.positions, "positions", torch.int32, (N,))
+    _call("ms_pooled_attention", q.data_ptr(), q.stride(0) if N > 1 else q.shape[1], k.data_ptr(), v.data_ptr(),
+          kv.block_table.data_ptr(), _ptr(pk), _ptr(pv), _ptr(ptab), kv.block_table.shape[1], _ptr(kv.table_rows),
+          _ptr(ctx.n_live_tokens), ctx.token_req.data_ptr(), ctx.positions.data_ptr(), _ptr(inv_freq_v), out.data_ptr(),
+          num_heads * dv, N, num_heads, nkv, d, dv, page_size, float(scale), int(size), int(pool), _code(q.dtype), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ gated activations
+def clamped_glu(gu: torch.Tensor, out: torch.Tensor, limit: float, alpha: float = 1.702) -> torch.Tensor:
+    """gu [N, 2F] with gate and up interleaved: g = min(g, limit), u = clamp(u, -limit, limit),
+    out = g * sigmoid(alpha g) * (u + 1), [N, F]."""
+    F = gu.shape[1] // 2
+    s_in = _rows2d(gu, "gu", None, 2 * F)
+    s_out = _rows2d(out, "out", gu.dtype, F)
+    if out.shape[0] != gu.shape[0]:
+        raise ValueError("out has one row per row of gu")
+    _call("ms_clamped_glu", gu.data_ptr(), s_in, out.data_ptr(), s_out, gu.shape[0], F, float(limit), float(alpha),
+          _code(gu.dtype), _stream())
+    return out
+
+
+def scaled_swiglu(gu: torch.Tensor, out: torch.Tensor, factor: Optional[torch.Tensor] = None,
+                  row_item: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """gu [rows, 2F] with gate and up interleaved: out = silu(s g) * (s u) with s = factor[row_item[p]] for row p
+    (factor[p] without ``row_item``; 1 without ``factor``); rows with a negative ``row_item`` are left alone."""
+    F = gu.shape[1] // 2
+    s_in = _rows2d(gu, "gu", None, 2 * F)
+    s_out = _rows2d(out, "out", gu.dtype, F)
+    n = gu.shape[0]
+    if out.shape[0] != n:
+        raise ValueError("out has one row per row of gu")
+    if factor is not None:
+        _check(factor, "factor", torch.float32)
+    if row_item is not None:
+        _check(row_item, "row_item", torch.int32)
+        if row_item.numel() < n:
+            raise ValueError("row_item names an item for every row")
+    _call("ms_scaled_swiglu", gu.data_ptr(), s_in, _ptr(factor), _ptr(row_item), out.data_ptr(), s_out, n, F,
+          _code(gu.dtype), _stream())
     return out

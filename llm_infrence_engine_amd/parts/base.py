@@ -58,10 +58,14 @@ class PageTensor:
 @dataclass(frozen=True)
 class CacheNeed:
     """What a mixer keeps per token in pages: one or more tensors, for all tokens of a request (``window``
-    None) or the last ``window`` of them.  Runs with equal needs share a group of the cache manager."""
+    None) or the last ``window`` of them.  Runs with equal needs share a group of the cache manager.
+    ``stride`` = s > 1: the pages hold one entry for every *whole block* of s tokens instead of one per token
+    (entry b belongs to the tokens b s .. b s + s - 1 and is stored with the block's last token), so a request
+    of L tokens holds floor(L / s) entries there.  A mixer that keeps both kinds returns a tuple of needs."""
 
     tensors: Tuple[PageTensor, ...]
     window: Optional[int] = None
+    stride: int = 1
 
     def __post_init__(self):
         names = [t.name for t in self.tensors]
@@ -69,6 +73,8 @@ class CacheNeed:
             raise ValueError("a cache need names at least one page tensor, each name once")
         if self.window is not None and self.window <= 0:
             raise ValueError("window must be positive")
+        if self.stride < 1 or (self.stride > 1 and self.window is not None):
+            raise ValueError("stride must be at least 1, and entries kept per block of tokens have no window")
 
     def values_per_token(self) -> int:
         return sum(t.heads * t.width for t in self.tensors)
@@ -104,6 +110,8 @@ class KVView:
     store: bool = True                   # False: the run reads another run's cache and writes nothing
     window: Optional[int] = None
     table_rows: Optional[torch.Tensor] = None   # int32 [R]; None: request r reads row r
+    stride: int = 1                      # tokens per entry of these pages (``CacheNeed.stride``)
+    more: tuple = ()                     # the views of the mixer's further cache needs, in the order it stated them
 
     def pages_of(self, r: int) -> torch.Tensor:
         """The block-table row of the step's request ``r`` (for parts written in plain tensor code)."""
@@ -235,7 +243,8 @@ class Mixer(Part):
         ``graph_safe = True`` or ``"decode"``."""
         return self.state_need() is None
 
-    def cache_need(self) -> Optional[CacheNeed]:
+    def cache_need(self):
+        """None, a ``CacheNeed``, or a tuple of them (the run's view of the first carries the others in ``more``)."""
         return None
 
     def state_need(self):
@@ -344,6 +353,8 @@ class Block(Part):
         needs = self._caching_mixers()
         if len(needs) <= 1:
             return next(iter(needs.values()), None)
+        if any(isinstance(n, (tuple, list)) for n in needs.values()):
+            raise ValueError("a mixer with several cache needs must be the only caching mixer of its layer")
         windows = {n.window for n in needs.values()}
         if len(windows) > 1:
             raise ValueError(f"the caching mixers {sorted(needs)} of one layer keep their tokens for different spans "
@@ -410,6 +421,22 @@ class Block(Part):
         raise NotImplementedError
 
 
+class Scale(Part):
+    """A float vector that a sublayer's result is multiplied by, element by element, on its way into the residual
+    stream (``vector`` after ``load``)."""
+
+    vector: torch.Tensor = None
+
+
+class TokenInput(Part):
+    """Something a layer adds to the residual stream that reads the step's token ids again."""
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, delta: Optional[torch.Tensor] = None,
+                delta_scale: Optional[torch.Tensor] = None) -> None:
+        """x [N, H] (float) <- x (+ delta_scale o delta) + what the part makes of that sum and the tokens, in place."""
+        raise NotImplementedError
+
+
 class PassEntry(Part):
     """What happens to the residual stream right before a pass over a stretch of layers that is walked several times."""
 
@@ -437,7 +464,7 @@ class Head(Part):
 # ------------------------------------------------------------------------------------------------ registries
 _REGISTRIES: Dict[str, Dict[str, type]] = {
     "norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "filter": {}, "block": {}, "embedding": {}, "head": {},
-    "pass_entry": {},
+    "pass_entry": {}, "scale": {}, "token_input": {},
 }
 
 

@@ -71,6 +71,38 @@ class SandwichResidual(Block):
         return None
 
 
+class ScaledPreNormResidual(Block):
+    """x <- x + s1 o mixer(norm1(x));  x <- x + s2 o feed_forward(norm2(x));  then, if the layer has one, the token's own
+    input (``token_input``) into x.  s1, s2 (``mixer_scale``, ``feed_forward_scale``; optional) are stored vectors.  Every
+    scaled sum rides on the kernel that reads x next: the second norm, the token input, or a sum of its own.  Without a
+    feed-forward the layer is its first line (and the token input)."""
+
+    takes = {"position": "position", "mixer_norm": "norm", "mixer": "mixer", "mixer_scale": "scale",
+             "feed_forward_norm": "norm", "feed_forward": "feed_forward", "feed_forward_scale": "scale",
+             "token_input": "token_input"}
+    optional = ("position", "mixer_scale", "feed_forward_norm", "feed_forward", "feed_forward_scale", "token_input")
+
+    @staticmethod
+    def _normed(norm, x, delta, scale):
+        if delta is not None and scale is not None and not getattr(norm, "takes_delta_scale", False):
+            ops.layer_norm(x, None, 0.0, None, delta=delta, delta_scale=scale)      # the scaled sum alone
+            return norm.forward(x)
+        return norm.forward(x, delta=delta, delta_scale=scale) if scale is not None else norm.forward(x, delta=delta)
+
+    def forward(self, x, pending, ctx, kv, state):
+        y = self.mixer.forward(self.mixer_norm.forward(x, delta=pending), ctx, kv, state)
+        scale = self.mixer_scale.vector if self.mixer_scale is not None else None
+        if self.feed_forward is not None:
+            y = self.feed_forward.forward(self._normed(self.feed_forward_norm, x, y, scale), ctx)
+            scale = self.feed_forward_scale.vector if self.feed_forward_scale is not None else None
+        if self.token_input is not None:
+            self.token_input.forward(x, ctx, delta=y, delta_scale=scale)
+        else:
+            ops.layer_norm(x, None, 0.0, None, delta=y, delta_scale=scale)
+        return None
+
+
 register_part("block", "pre_norm_residual", PreNormResidual)
+register_part("block", "pre_norm_scaled_residual", ScaledPreNormResidual)
 register_part("block", "sandwich_residual", SandwichResidual)
 register_part("block", "parallel_residual", ParallelResidual)

@@ -7,25 +7,33 @@ import torch
 
 from ..kernels import linear, ops
 from ..weights.spec import TensorSpec
-from .base import Embedding, Head, PassEntry, register_part
+from .base import Embedding, Head, PassEntry, build_part, register_part
 
 
 class TokenEmbedding(Embedding):
-    def __init__(self, prefix: str, vocab_size: int, hidden_size: int, name: str = "weight", scale: float = 1.0):
-        """``scale``: every row is multiplied by it on its way into the float residual stream."""
+    def __init__(self, prefix: str, vocab_size: int, hidden_size: int, name: str = "weight", scale: float = 1.0, norm=None):
+        """``scale``: every row is multiplied by it on its way into the float residual stream.  ``norm``: the
+        ``PartSpec`` of a norm that the rows pass right after (one with ``normalize_``), or None."""
         self.prefix, self.vocab_size, self.hidden_size, self.name = prefix, vocab_size, hidden_size, name
         self.scale = float(scale)
+        self.norm = build_part("norm", norm) if norm is not None else None
+        if self.norm is not None and not hasattr(self.norm, "normalize_"):
+            raise ValueError(f"the norm {norm.kind!r} cannot be applied in place to the embedding's rows")
 
     def tensor_specs(self):
-        return [TensorSpec(self.prefix + self.name, (self.vocab_size, self.hidden_size))]
+        return [TensorSpec(self.prefix + self.name, (self.vocab_size, self.hidden_size))] + \
+            (self.norm.tensor_specs() if self.norm is not None else [])
 
     def load(self, get, rt):
         self.rt = rt
-        self.weight = get(self.tensor_specs()[0])
+        self.weight = get(TokenEmbedding.tensor_specs(self)[0])
+        if self.norm is not None:
+            self.norm.load(get, rt)
 
     def forward(self, ctx):
         out = self.rt.empty(ctx.num_tokens, self.hidden_size, dtype=torch.float32)
-        return ops.embed(ctx.token_ids, self.weight, out, self.scale)
+        ops.embed(ctx.token_ids, self.weight, out, self.scale)
+        return self.norm.normalize_(out) if self.norm is not None else out
 
 
 class LMHead(Head):

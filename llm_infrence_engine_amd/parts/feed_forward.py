@@ -65,5 +65,32 @@ class DenseAct(FeedForward):
         return linear.linear_residual(u, self.w_down, None, x)
 
 
+class ClampedGLU(FeedForward):
+    """down(g * sigmoid(alpha g) * (u + 1)) with g = min(gate(x), limit) and u = clamp(up(x), -limit, limit); no biases.
+    Gate and up are one packed product (rows interleaved); clamps and activation are float."""
+
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, limit: float, alpha: float = 1.702,
+                 gate_name: str = "gate", up_name: str = "up", down_name: str = "down"):
+        self.prefix, self.hidden_size, self.intermediate_size = prefix, hidden_size, intermediate_size
+        self.limit, self.alpha = float(limit), float(alpha)
+        self.gate_name, self.up_name, self.down_name = gate_name, up_name, down_name
+
+    def tensor_specs(self):
+        p, H, I = self.prefix, self.hidden_size, self.intermediate_size
+        return [TensorSpec(p + self.gate_name, (I, H)), TensorSpec(p + self.up_name, (I, H)), TensorSpec(p + self.down_name, (H, I))]
+
+    def load(self, get, rt):
+        self.rt = rt
+        g, u, d = (get(s) for s in self.tensor_specs())
+        self.w_gate_up = linear.interleave_rows(g, u)
+        self.w_down = linear.prepare_weight(d)
+
+    def forward(self, h, ctx):
+        gu = linear.linear(h, self.w_gate_up)
+        act = ops.clamped_glu(gu, self.rt.empty(gu.shape[0], self.intermediate_size), self.limit, self.alpha)
+        return linear.linear(act, self.w_down)
+
+
 register_part("feed_forward", "swiglu", SwiGLU)
+register_part("feed_forward", "clamped_glu", ClampedGLU)
 register_part("feed_forward", "dense_act", DenseAct)

@@ -13,7 +13,8 @@ import torch
 from ..config.spec import ModelSpec
 from ..weights.reader import CheckpointReader, place
 from ..weights.spec import TensorSpec
-from . import attention, blocks, delta, ends, experts, feed_forward, filters, latent, norms, positions, scan  # noqa: F401  (register the built-in parts)
+from . import (attention, blocks, delta, ends, experts, feed_forward, filters, latent, mingru, norms,  # noqa: F401
+               pooled_attention, positions, scan, side)      # (register the built-in parts)
 from .base import KVView, Runtime, StateView, StepContext, build_part, part_class, weakest
 
 

@@ -70,4 +70,33 @@ class RMSNorm(Norm):
         return linear.LazyNorm(x, self.weight, self.eps, self.rt.dtype, rows)
 
 
+class LayerNorm(Norm):
+    """y = weight * (x - mean x) / sqrt(mean (x - mean x)^2 + eps): a weight and no bias, computed in float on the float
+    residual stream.  ``forward`` also takes ``delta_scale``, a float vector the addend is multiplied by, element by
+    element, on its way into x (a layer's scale)."""
+
+    takes_delta_scale = True
+
+    def __init__(self, prefix: str, size: int, eps: float, name: str = "weight"):
+        self.prefix, self.size, self.eps, self.name = prefix, size, float(eps), name
+
+    def tensor_specs(self):
+        return [TensorSpec(self.prefix + self.name, (self.size,), "norm")]
+
+    def load(self, get, rt):
+        self.rt = rt
+        self.weight = get(self.tensor_specs()[0])
+
+    def forward(self, x, delta=None, rows=None, write_back=True, delta_scale=None):
+        n = x.shape[0] if rows is None else rows.numel()
+        out = self.rt.empty(n, self.size)
+        return ops.layer_norm(x, self.weight, self.eps, out, delta=delta, delta_scale=delta_scale, rows=rows,
+                              write_back=write_back)
+
+    def normalize_(self, x):
+        """The rows of the float stream x take their own norm, in place."""
+        return ops.layer_norm(x, self.weight, self.eps, x)
+
+
 register_part("norm", "rms_norm", RMSNorm)
+register_part("norm", "layer_norm", LayerNorm)
