@@ -170,7 +170,8 @@ class CacheManager:
 
     def capacity_tokens(self) -> int:
         """Tokens one request could hold if it had the smallest pool to itself."""
-        return min(self.max_len, self.num_pages * self.page_size) if self.groups else self.max_len
+        return min([self.max_len] + [n * self.page_size * g.key.stride + g.key.stride - 1
+                                     for g, n in zip(self.groups, self.pages_per_group)])
 
     # ------------------------------------------------------------------ pages
     def _first_needed(self, g: CacheGroup, computed: int) -> int:
