@@ -1,5 +1,5 @@
 """Named config.json contents for the random-weights mode: the shapes the published Qwen2.5 checkpoints
-have, the two tiny ones the tests use and two Gemadra and two Gidurax shapes of the same widths, so that ``--random-config 0.5b``
+have, the two tiny ones the tests use and two Gemadra, two Gidurax and two Kuvazen shapes of the same widths, so that ``--random-config 0.5b``
 needs no file.  These are data
 of the kind a config.json holds; no part or kernel reads them.
 """
@@ -69,6 +69,30 @@ PRESETS["gidurax-7b"] = _gidurax(
     {"heads": 28, "kv_heads": 14, "dim": 128, "vdim": 128, "conv": 4},
     {"heads": 28, "kv_heads": 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "q_temp": {"coef": 0.25, "every": 256}},
     (7104, 16, 2, 3, 7104), vocab=152064)
+
+
+def _kuvazen(width, ff, layers, gru_width, attention, experts, side, vocab=151936):
+    """``layers`` layers in the order minGRU, attention, minGRU, attention; the second and third with routed experts
+    (``experts``: (expert ff, experts, top)), the others with the dense clamped feed-forward."""
+    ef, n, top = experts
+    routed = {"kind": "moe", "expert": {"ff": ef}, "router": {"experts": n, "top": top}}
+    kinds = [("mingru", {"width": gru_width}), ("attention", attention)]
+    return {"architecture": "Kuvazen", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "token_side": {"dim": side},
+            "layers": [{"type": kinds[i % 2][0], "mixer": dict(kinds[i % 2][1]),
+                        "mlp": dict(routed) if i % 4 in (1, 2) else {"kind": "dense", "ff": ff, "limit": 7.0}} for i in range(layers)]}
+
+
+# Kuvazen at the same widths: gated dense feed-forwards of the Qwen2 shapes' size, routed ones whose three chosen experts
+# of sixteen have as many weights together; a window of 256 tokens and blocks of 16, so that a 2,048-token prompt sees
+# both tokens and blocks
+PRESETS["kuvazen-0.5b"] = _kuvazen(
+    896, 4864, 24, 1792,
+    {"heads": 14, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 64 ** -0.5, "mask": {"size": 256, "pool": 16},
+     "rot": {"base": 10000.0, "dims": 64}}, (1600, 16, 3), 64)
+PRESETS["kuvazen-7b"] = _kuvazen(
+    3584, 18944, 28, 7168,
+    {"heads": 28, "kv_heads": 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 256, "pool": 16},
+     "rot": {"base": 10000.0, "dims": 128}}, (6336, 16, 3), 256, vocab=152064)
 
 
 def preset(name: str) -> dict:

@@ -258,12 +258,11 @@ int ms_moe_combine(const float* part, const int* ids, const float* weights, cons
                    const void* shared, int shared_dtype, const float* gate, long long gate_stride, float* out,
                    int n_tokens, int top, int n_experts, int hidden, int dtype, hipStream_t stream);   // weights null: all 1
 
-// ---- layer norm and the token's side input (csrc/layer_norm.hip)
+// ---- layer norm and the gate of a token's side input (csrc/layer_norm.hip)
 int ms_layer_norm(float* x, const void* delta, int delta_dtype, const float* dscale, const float* w, const int* rows,
                   void* out, int n_rows, int H, float eps, int write_back, int out_dtype, hipStream_t stream);
-int ms_token_side(float* x, const void* delta, int delta_dtype, const float* dscale, const int* token_ids, const void* table,
-                  long long table_stride, int part, const void* G, const void* P, const float* w, int n_tokens, int H, int d,
-                  float eps, int dtype, hipStream_t stream);
+int ms_side_gate(const void* z, long long z_stride, const int* token_ids, const void* table, long long table_stride, int part,
+                 void* out, int n_tokens, int d, int dtype, hipStream_t stream);
 // ---- minGRU (csrc/mingru.hip)
 int ms_mingru_scan(const void* zxg, long long in_stride, const float* bz, const float* bx, float* state, const int* q_start,
                    const int* state_slots, void* out, long long out_stride, int n_requests, int C, int long_portions,
@@ -271,17 +270,25 @@ int ms_mingru_scan(const void* zxg, long long in_stride, const float* bz, const 
 // ---- window + pooled blocks attention (csrc/pooled_attention.hip)
 int ms_pairs_rotate_store(void* qkv, long long stride, const int* positions, const float* inv_freq, const float* inv_freq_v,
                           const int* slots, void* k_pages, void* v_pages, int n_tokens, int num_heads, int num_kv_heads,
-                          int head_dim, int value_dim, int rot_dims, int page_size, int dtype, hipStream_t stream);
+                          int head_dim, int value_dim, int rot_dims, int page_size, int v_transposed, int dtype,
+                          hipStream_t stream);
 int ms_pool_store(const void* k_pages, const void* v_pages, const int* table, int table_stride, const int* table_rows,
                   const int* token_req, const int* positions, const int* pool_slots, void* pk_pages, void* pv_pages,
-                  int n_tokens, int num_kv_heads, int head_dim, int value_dim, int page_size, int pool, int dtype,
-                  hipStream_t stream);
+                  int n_tokens, int num_kv_heads, int head_dim, int value_dim, int page_size, int pool, int v_transposed,
+                  int dtype, hipStream_t stream);
 int ms_pooled_attention(const void* q, long long q_stride, const void* k_pages, const void* v_pages, const int* table,
                         const void* pk_pages, const void* pv_pages, const int* pool_table, int table_stride,
                         const int* table_rows, const int* n_live_tokens, const int* token_req, const int* positions,
                         const float* inv_freq_v, void* out, long long out_stride, int n_tokens, int num_heads,
                         int num_kv_heads, int head_dim, int value_dim, int page_size, float scale, int size, int pool,
-                        int dtype, hipStream_t stream);
+                        int v_transposed, int dtype, hipStream_t stream);
+// the same on the matrix cores (csrc/attention_mfma.hip): bfloat16, value pages transposed, keys and values of one size
+int ms_pooled_attention_mfma(const void* q, long long q_stride, const void* k_pages, const void* vt_pages,
+                             const int* block_table, const void* pk_pages, const void* pvt_pages, const int* pool_table,
+                             int table_stride, const int* table_rows, const int* q_start, const int* context_lens,
+                             const float* turn_back, void* out, long long out_stride, int n_requests, int n_tokens,
+                             int max_q_len, int num_heads, int num_kv_heads, int head_dim, int page_size, float scale,
+                             int window, int pool, hipStream_t stream);
 // ---- gated activations (csrc/glu.hip)
 int ms_clamped_glu(const void* gu, long long in_stride, void* out, long long out_stride, int n_rows, int F, float limit,
                    float alpha, int dtype, hipStream_t stream);

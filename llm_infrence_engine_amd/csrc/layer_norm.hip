@@ -1,12 +1,13 @@
-// Layer norm with a weight and no bias on the float residual stream, the scaled sum that precedes it, and a token's
-// own side input into the stream.
+// Layer norm with a weight and no bias on the float residual stream, the scaled sum that precedes it, and the gate of a
+// token's own side input into the stream.
 //   v = x[row] (+ scale o delta[row]);   out = w o (v - mean v) / sqrt(mean (v - mean v)^2 + eps)
 // The row is held in LDS between the passes (mean, then the mean of the squared deviations, as the norm is defined; no
-// E[v^2] - E[v]^2), so out may be x itself.  Everything is float; out is rounded once.
+// E[v^2] - E[v]^2), so out may be x itself.  Everything is float; out is rounded once.  Without a weight the kernel is
+// the scaled sum alone, and out (if given) takes the summed row rounded to its type: the operand of a product that reads
+// the stream itself.
 //
-// Side input of layer i for token n (c = side_table[token, i d .. i d + d - 1], d small):
-//   g = gelu_tanh(G v) o c;   y = P g;   x[n] = v + y / sqrt(mean y^2 + eps) o w_side
-// one block per token: G [d, H] row by row over the waves, P [H, d] a row per thread.
+// ms_side_gate: g[n, j] = gelu_tanh(z[n, j]) * table[token[n], part d + j], what stands between the two small products
+// of a layer's side input (z = G x before it, y = P g after it).
 #include "common.h"
 #include "api.h"
 
@@ -45,6 +46,7 @@ layer_norm_kernel(float* __restrict__ x, const TD* __restrict__ delta, const flo
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     if (delta && write_back && !same) xr[i] = row[i];
     if (w) o[i] = from_float<TO>((row[i] - mean) * inv * w[i]);
+    else if (out) o[i] = from_float<TO>(row[i]);
   }
 }
 
@@ -52,40 +54,15 @@ __device__ __forceinline__ float gelu_tanh(float z) {
   return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
 
-template <typename T, typename TD>
-__global__ void __launch_bounds__(LN_THREADS)
-token_side_kernel(float* __restrict__ x, const TD* __restrict__ delta, const float* __restrict__ dscale,
-                  const int* __restrict__ token_ids, const T* __restrict__ table, size_t table_stride, int part,
-                  const T* __restrict__ G, const T* __restrict__ P, const float* __restrict__ w, int H, int d, float eps) {
-  extern __shared__ float sh[];
-  float* row = sh;            // [H]
-  float* y = sh + H;          // [H]
-  float* g = sh + 2 * H;      // [d]
-  __shared__ float red[16];
-  const size_t n = blockIdx.x;
-  float* xr = x + n * H;
-  load_row<TD>(row, xr, delta ? delta + n * H : nullptr, dscale, H);
-  __syncthreads();
-  const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE, waves = blockDim.x / MS_WAVE;
-  const T* c = table + (size_t)token_ids[n] * table_stride + (size_t)part * d;
-  for (int j = wave; j < d; j += waves) {
-    const T* gj = G + (size_t)j * H;
-    float dot = 0.f;
-    for (int i = lane; i < H; i += MS_WAVE) dot = fmaf(to_float(gj[i]), row[i], dot);
-    dot = wave_sum(dot);
-    if (lane == 0) g[j] = gelu_tanh(dot) * to_float(c[j]);
-  }
-  __syncthreads();
-  float q = 0.f;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    const T* pi = P + (size_t)i * d;
-    float v = 0.f;
-    for (int j = 0; j < d; ++j) v = fmaf(to_float(pi[j]), g[j], v);
-    y[i] = v;
-    q = fmaf(v, v, q);
-  }
-  const float inv = 1.0f / sqrtf(block_sum(q, red) / (float)H + eps);
-  for (int i = threadIdx.x; i < H; i += blockDim.x) xr[i] = row[i] + y[i] * inv * w[i];
+template <typename T>
+__global__ void __launch_bounds__(256)
+side_gate_kernel(const T* __restrict__ z, size_t z_stride, const int* __restrict__ token_ids, const T* __restrict__ table,
+                 size_t table_stride, int part, T* __restrict__ out, int n_tokens, int d) {
+  const long long item = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (item >= (long long)n_tokens * d) return;
+  const int n = (int)(item / d), j = (int)(item - (long long)n * d);
+  const float c = to_float(table[(size_t)token_ids[n] * table_stride + (size_t)part * d + j]);
+  out[(size_t)n * d + j] = from_float<T>(gelu_tanh(to_float(z[(size_t)n * z_stride + j])) * c);
 }
 
 }  // namespace
@@ -96,7 +73,7 @@ extern "C" int ms_layer_norm(float* x, const void* delta, int delta_dtype, const
                              const int* rows, void* out, int n_rows, int H, float eps, int write_back, int out_dtype,
                              hipStream_t stream) {
   if (n_rows <= 0) return MS_OK;
-  if (H <= 0 || (w != nullptr && out == nullptr)) return MS_BAD_ARG;
+  if (H <= 0 || (w != nullptr && out == nullptr)) return MS_BAD_ARG;   // w null with out: the summed rows' rounded copy
   if (H > 16384) return MS_UNSUPPORTED;
   const size_t lds = (size_t)H * sizeof(float);
 #define LAUNCH(TD, TO)                                                                                               \
@@ -111,22 +88,15 @@ extern "C" int ms_layer_norm(float* x, const void* delta, int delta_dtype, const
   return ms_launch_status();
 }
 
-// table [vocab, table_stride] and the matrices G [d, H], P [H, d] of `dtype`; token_ids int32 [N]; w float [H].
-extern "C" int ms_token_side(float* x, const void* delta, int delta_dtype, const float* dscale, const int* token_ids,
-                             const void* table, long long table_stride, int part, const void* G, const void* P,
-                             const float* w, int n_tokens, int H, int d, float eps, int dtype, hipStream_t stream) {
+// z [N, d] (rows z_stride apart), table [vocab, table_stride], out [N, d] of `dtype`; token_ids int32 [N].
+extern "C" int ms_side_gate(const void* z, long long z_stride, const int* token_ids, const void* table, long long table_stride,
+                            int part, void* out, int n_tokens, int d, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return MS_OK;
-  if (H <= 0 || d <= 0 || part < 0 || (long long)(part + 1) * d > table_stride) return MS_BAD_ARG;
-  if (2 * (size_t)H + d > 15000) return MS_UNSUPPORTED;     // 60 KB of LDS
-  const size_t lds = (2 * (size_t)H + d) * sizeof(float);
-#define LAUNCH(T, TD)                                                                                                \
-  token_side_kernel<T, TD><<<dim3(n_tokens), dim3(LN_THREADS), lds, stream>>>(                                       \
-      x, (const TD*)delta, dscale, token_ids, (const T*)table, (size_t)table_stride, part, (const T*)G, (const T*)P, w, H, d, eps)
-  const bool dbf = delta != nullptr && delta_dtype == MS_BF16;
-  if (delta != nullptr && delta_dtype != MS_BF16 && delta_dtype != MS_F32) return MS_BAD_ARG;
-  if (dtype == MS_F32) { if (dbf) LAUNCH(float, bf16); else LAUNCH(float, float); }
-  else if (dtype == MS_BF16) { if (dbf) LAUNCH(bf16, bf16); else LAUNCH(bf16, float); }
+  if (d <= 0 || part < 0 || (long long)(part + 1) * d > table_stride || z_stride < d) return MS_BAD_ARG;
+  const long long items = (long long)n_tokens * d;
+  dim3 grid((unsigned)((items + 255) / 256)), block(256);
+  if (dtype == MS_F32) side_gate_kernel<float><<<grid, block, 0, stream>>>((const float*)z, (size_t)z_stride, token_ids, (const float*)table, (size_t)table_stride, part, (float*)out, n_tokens, d);
+  else if (dtype == MS_BF16) side_gate_kernel<bf16><<<grid, block, 0, stream>>>((const bf16*)z, (size_t)z_stride, token_ids, (const bf16*)table, (size_t)table_stride, part, (bf16*)out, n_tokens, d);
   else return MS_BAD_ARG;
-#undef LAUNCH
   return ms_launch_status();
 }

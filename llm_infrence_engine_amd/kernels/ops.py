@@ -102,17 +102,19 @@ _SIGNATURES = {
     "ms_gelu": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
     "ms_moe_route": [_c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "ms_layer_norm": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
-    "ms_token_side": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
-                      _c_int, _c_float, _c_int, _c_ptr],
+    "ms_side_gate": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "ms_mingru_scan": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int,
                        _c_ptr],
     "ms_pairs_rotate_store": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
-                              _c_int, _c_int, _c_int, _c_int, _c_ptr],
+                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_pool_store": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
-                      _c_int, _c_int, _c_int, _c_int, _c_ptr],
+                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_pooled_attention": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
                             _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
-                            _c_int, _c_int, _c_ptr],
+                            _c_int, _c_int, _c_int, _c_ptr],
+    "ms_pooled_attention_mfma": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                                 _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
+                                 _c_int, _c_int, _c_ptr],
     "ms_clamped_glu": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_int, _c_int, _c_float, _c_float, _c_int, _c_ptr],
     "ms_scaled_swiglu": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_ptr],
     "ms_moe_tile_rows": [],
@@ -1392,7 +1394,8 @@ def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out:
                rows: Optional[torch.Tensor] = None, write_back: bool = True):
     """out[r] = weight * (v - mean v) / sqrt(mean (v - mean v)^2 + eps) with v = x[rows[r]] (+ delta_scale o delta[rows[r]]).
     x float32 [N, H] is the residual stream; with ``delta`` [N, H] the sum is written back to x (unless ``write_back`` is
-    False).  ``weight`` None: only the sum.  ``out`` may be x itself (float): the rows are normed in place."""
+    False).  ``weight`` None: only the sum, and ``out`` (if given) takes the summed rows rounded to its type.  ``out`` may
+    be x itself (float): the rows are normed in place."""
     _check(x, "x", torch.float32)
     N, H = x.shape
     n_rows = N
@@ -1401,6 +1404,7 @@ def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out:
         n_rows = rows.numel()
     if weight is not None:
         _check(weight, "weight", torch.float32, (H,))
+    if weight is not None or out is not None:
         _check(out, "out", None, (n_rows, H))
     dcode = 0
     if delta is not None:
@@ -1411,37 +1415,22 @@ def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out:
     elif delta_scale is not None:
         raise ValueError("a scale without an addend")
     _call("ms_layer_norm", x.data_ptr(), _ptr(delta), dcode, _ptr(delta_scale), _ptr(weight), _ptr(rows),
-          _ptr(out) if weight is not None else None, n_rows, H, float(eps), int(write_back),
-          _code(out.dtype) if weight is not None else F32, _stream())
+          _ptr(out), n_rows, H, float(eps), int(write_back), _code(out.dtype) if out is not None else F32, _stream())
     return out
 
 
-def token_side(x: torch.Tensor, token_ids: torch.Tensor, table: torch.Tensor, part: int, gate: torch.Tensor,
-               proj: torch.Tensor, weight: torch.Tensor, eps: float, delta: Optional[torch.Tensor] = None,
-               delta_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x[n] <- v + y / sqrt(mean y^2 + eps) o weight, with v = x[n] (+ delta_scale o delta[n]), c = table[token_ids[n],
-    part d : (part + 1) d], y = proj (gelu_tanh(gate v) o c).  x float32 [N, H]; table [V, parts d]; gate [d, H]; proj
-    [H, d]; weight float [H]."""
-    _check(x, "x", torch.float32)
-    N, H = x.shape
-    d = gate.shape[0]
-    _check(gate, "gate", table.dtype, (d, H))
-    _check(proj, "proj", table.dtype, (H, d))
+def side_gate(z: torch.Tensor, token_ids: torch.Tensor, table: torch.Tensor, part: int, out: torch.Tensor) -> torch.Tensor:
+    """out[n, j] = gelu_tanh(z[n, j]) * table[token_ids[n], part d + j] for z [N, d] (rows may be slices); table [V, parts d]."""
+    N, d = z.shape
+    zs = _rows2d(z, "z", table.dtype)
     _check(table, "table")
     if table.dim() != 2 or (part + 1) * d > table.shape[1] or part < 0:
         raise ValueError(f"part {part} of {d} entries is not within the table's rows of {table.shape[1]}")
     _check(token_ids, "token_ids", torch.int32, (N,))
-    _check(weight, "weight", torch.float32, (H,))
-    dcode = 0
-    if delta is not None:
-        _check(delta, "delta", None, (N, H))
-        dcode = _code(delta.dtype)
-        if delta_scale is not None:
-            _check(delta_scale, "delta_scale", torch.float32, (H,))
-    _call("ms_token_side", x.data_ptr(), _ptr(delta), dcode, _ptr(delta_scale), token_ids.data_ptr(), table.data_ptr(),
-          table.shape[1], int(part), gate.data_ptr(), proj.data_ptr(), weight.data_ptr(), N, H, d, float(eps),
-          _code(table.dtype), _stream())
-    return x
+    _check(out, "out", table.dtype, (N, d))
+    _call("ms_side_gate", z.data_ptr(), zs, token_ids.data_ptr(), table.data_ptr(), table.shape[1], int(part), out.data_ptr(),
+          N, d, _code(table.dtype), _stream())
+    return out
 
 
 # ------------------------------------------------------------------------------------------------ minGRU
@@ -1470,12 +1459,15 @@ def mingru_scan(zxg: torch.Tensor, bias_z: Optional[torch.Tensor], bias_x: Optio
 
 # ------------------------------------------------------------------------------------------------ window + pooled blocks
 def _token_pages(kv, names=("k", "v")):
+    """(key pages [P, heads, page, d], value pages, value size, whether the value pages are [P, heads, dv, page])."""
     k, v = kv.pages[names[0]], kv.pages[names[1]]
-    if kv.transposed.get(names[0]) or kv.transposed.get(names[1]):
-        raise ValueError("these kernels read pages as [page, head, slot, width]")
+    if kv.transposed.get(names[0]):
+        raise ValueError("these kernels read key pages as [page, head, slot, width]")
+    flipped = bool(kv.transposed.get(names[1]))
     _check(k, "k pages")
-    _check(v, "v pages", k.dtype, (k.shape[0], k.shape[1], k.shape[2], None))
-    return k, v
+    P, nkv, page, _ = k.shape
+    _check(v, "v pages", k.dtype, (P, nkv, None, page) if flipped else (P, nkv, page, None))
+    return k, v, (v.shape[2] if flipped else v.shape[3]), flipped
 
 
 def pairs_rotate_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
@@ -1493,44 +1485,49 @@ def pairs_rotate_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, hea
     store = kv is not None and kv.store
     k = v = None
     page_size = 1
+    flipped = False
     if store:
-        k, v = _token_pages(kv)
+        k, v, dv, flipped = _token_pages(kv)
         _check(k, "k pages", qkv.dtype, (None, num_kv_heads, None, head_dim))
-        _check(v, "v pages", qkv.dtype, (None, num_kv_heads, None, value_dim))
+        if dv != value_dim:
+            raise ValueError(f"the value pages hold values of {dv} entries, not {value_dim}")
         _check(kv.slot_mapping, "slot_mapping", torch.int32, (N,))
         page_size = k.shape[2]
     _call("ms_pairs_rotate_store", qkv.data_ptr(), stride, positions.data_ptr(), inv_freq.data_ptr(), inv_freq_v.data_ptr(),
           kv.slot_mapping.data_ptr() if store else None, _ptr(k), _ptr(v), N, num_heads, num_kv_heads, head_dim, value_dim,
-          rot_dims, page_size, _code(qkv.dtype), _stream())
+          rot_dims, page_size, int(flipped), _code(qkv.dtype), _stream())
     return qkv
 
 
 def pool_store(kv, pooled, ctx, pool: int) -> None:
     """For every token of the step that ends a block of ``pool`` tokens (its slot in ``pooled`` is not negative): the means
     of the block's keys and values, read back from ``kv``'s pages, go into ``pooled``'s pages "k" and "v"."""
-    k, v = _token_pages(kv)
-    pk, pv = _token_pages(pooled)
+    k, v, dv, flipped = _token_pages(kv)
+    pk, pv, pdv, pflipped = _token_pages(pooled)
     P, nkv, page_size, d = k.shape
-    dv = v.shape[3]
     _check(pk, "pooled k", k.dtype, (None, nkv, page_size, d))
-    _check(pv, "pooled v", k.dtype, (None, nkv, page_size, dv))
+    if pdv != dv or pflipped != flipped:
+        raise ValueError("the pooled value pages must have the size and the layout of the tokens' value pages")
     N = ctx.num_tokens
     _check(pooled.slot_mapping, "pooled slots", torch.int32, (N,))
     _check(kv.block_table, "block_table", torch.int32)
     _call("ms_pool_store", k.data_ptr(), v.data_ptr(), kv.block_table.data_ptr(), kv.block_table.shape[1],
           _ptr(kv.table_rows), ctx.token_req.data_ptr(), ctx.positions.data_ptr(), pooled.slot_mapping.data_ptr(),
-          pk.data_ptr(), pv.data_ptr(), N, nkv, d, dv, page_size, int(pool), _code(k.dtype), _stream())
+          pk.data_ptr(), pv.data_ptr(), N, nkv, d, dv, page_size, int(pool), int(flipped), _code(k.dtype), _stream())
 
 
 def pooled_attention(q: torch.Tensor, kv, pooled, ctx, out: torch.Tensor, num_heads: int, scale: float, size: int,
-                     pool: int, inv_freq_v: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     pool: int, inv_freq_v: Optional[torch.Tensor] = None, turn_back: Optional[torch.Tensor] = None,
+                     matrix_cores: Optional[bool] = None) -> torch.Tensor:
     """out[n, h] = softmax over the last ``size`` tokens up to n's position and over the pooled entry of every block of
     ``pool`` tokens that lies wholly before that window (block b: b pool + pool - 1 <= position - size), one softmax for
     both; tokens from ``kv``'s pages, block b from entry b of ``pooled``'s (None: no blocks).  With ``inv_freq_v`` the
-    output's entries 2m, 2m + 1 are turned by -position * inv_freq_v[m].  q [N, >= nh d] row slices; out [N, nh dv]."""
-    k, v = _token_pages(kv)
+    output's entries 2m, 2m + 1 are turned by -position * inv_freq_v[m].  q [N, >= nh d] row slices; out [N, nh dv].
+    bfloat16 with transposed value pages, keys and values of one size that the matrix-core kernel has and pooled blocks
+    goes there (``matrix_cores``: None decides by that, True insists, False keeps to the vector ALUs); it takes the cosines
+    and sines of the angles from ``turn_back`` (``rope_table(positions, inv_freq_v)``), made here if not given."""
+    k, v, dv, flipped = _token_pages(kv)
     P, nkv, page_size, d = k.shape
-    dv = v.shape[3]
     _check(q, "q", k.dtype, contiguous=False)
     N = q.shape[0]
     if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < num_heads * d:
@@ -1540,9 +1537,10 @@ def pooled_attention(q: torch.Tensor, kv, pooled, ctx, out: torch.Tensor, num_he
         raise ValueError(f"{num_heads} query heads cannot share {nkv} key/value heads")
     pk = pv = ptab = None
     if pooled is not None and pool > 0:
-        pk, pv = _token_pages(pooled)
+        pk, pv, pdv, pflipped = _token_pages(pooled)
         _check(pk, "pooled k", k.dtype, (None, nkv, page_size, d))
-        _check(pv, "pooled v", k.dtype, (None, nkv, page_size, dv))
+        if pdv != dv or pflipped != flipped:
+            raise ValueError("the pooled value pages must have the size and the layout of the tokens' value pages")
         ptab = pooled.block_table
         _check(ptab, "pooled table", torch.int32, tuple(kv.block_table.shape))
     else:
@@ -1551,10 +1549,30 @@ def pooled_attention(q: torch.Tensor, kv, pooled, ctx, out: torch.Tensor, num_he
         _check(inv_freq_v, "inv_freq_v", torch.float32, (dv // 2,))
     _check(ctx.token_req, "token_req", torch.int32, (N,))
     _check(ctx.positions, "positions", torch.int32, (N,))
+    can = (q.dtype == torch.bfloat16 and flipped and dv == d and pool > 0 and attention_mfma_supported(d, page_size)
+           and q.data_ptr() % 16 == 0 and (N == 1 or q.stride(0) % 8 == 0))
+    if matrix_cores and not can:
+        raise UnsupportedShape("the matrix-core kernel takes bfloat16, transposed value pages of the keys' size (32, 64 or "
+                               "128) and pages of a multiple of 16 tokens")
+    if can and matrix_cores is not False:
+        R = ctx.num_requests
+        _check(ctx.q_start, "q_start", torch.int32, (R + 1,))
+        _check(ctx.context_lens, "context_lens", torch.int32, (R,))
+        if inv_freq_v is not None and turn_back is None:
+            turn_back = rope_table(ctx.positions, inv_freq_v)
+        if turn_back is not None:
+            _check(turn_back, "turn_back", torch.float32, (N, d // 2, 2))
+        _call("ms_pooled_attention_mfma", q.data_ptr(), q.stride(0) if N > 1 else q.shape[1], k.data_ptr(), v.data_ptr(),
+              kv.block_table.data_ptr(), pk.data_ptr(), pv.data_ptr(), ptab.data_ptr(), kv.block_table.shape[1],
+              _ptr(kv.table_rows), ctx.q_start.data_ptr(), ctx.context_lens.data_ptr(), _ptr(turn_back), out.data_ptr(),
+              num_heads * dv, R, N, max(1, ctx.max_q_len), num_heads, nkv, d, page_size, float(scale), int(size), int(pool),
+              _stream())
+        return out
     _call("ms_pooled_attention", q.data_ptr(), q.stride(0) if N > 1 else q.shape[1], k.data_ptr(), v.data_ptr(),
           kv.block_table.data_ptr(), _ptr(pk), _ptr(pv), _ptr(ptab), kv.block_table.shape[1], _ptr(kv.table_rows),
           _ptr(ctx.n_live_tokens), ctx.token_req.data_ptr(), ctx.positions.data_ptr(), _ptr(inv_freq_v), out.data_ptr(),
-          num_heads * dv, N, num_heads, nkv, d, dv, page_size, float(scale), int(size), int(pool), _code(q.dtype), _stream())
+          num_heads * dv, N, num_heads, nkv, d, dv, page_size, float(scale), int(size), int(pool), int(flipped),
+          _code(q.dtype), _stream())
     return out
 
 

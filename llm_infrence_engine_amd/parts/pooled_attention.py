@@ -63,7 +63,10 @@ class PooledWindowAttention(Mixer):
         self.inv_freq_v = f.to(torch.float32).to(rt.device)
 
     def cache_need(self):
-        tensors = (PageTensor("k", self.num_kv_heads, self.head_dim), PageTensor("v", self.num_kv_heads, self.value_dim))
+        # in bfloat16 the matrix-core kernel reads value pages (of tokens and of blocks) as an operand as they lie,
+        # transposed, which it can for values of the keys' size in pages of a multiple of 16 tokens
+        flip = dict(transpose_at=16, transpose_in=torch.bfloat16) if self.value_dim == self.head_dim else {}
+        tensors = (PageTensor("k", self.num_kv_heads, self.head_dim), PageTensor("v", self.num_kv_heads, self.value_dim, **flip))
         return (CacheNeed(tensors, window=max(self.size, self.pool)), CacheNeed(tensors, stride=self.pool))
 
     def forward(self, h, ctx, kv, state):
@@ -76,8 +79,15 @@ class PooledWindowAttention(Mixer):
         if kv.store:
             ops.pool_store(kv, pooled, ctx, self.pool)
         out = self.rt.empty(ctx.num_tokens, nh * dv)
+        turn_back = None
+        if self.rotate_values and qkv.dtype == torch.bfloat16 and kv.transposed.get("v"):
+            # cosines and sines of the step's positions: worked out by the first layer that comes here, shared by the others
+            key = ("rotary_pairs", dv, self.value_theta)
+            turn_back = ctx.shared.get(key)
+            if turn_back is None:
+                turn_back = ctx.shared[key] = ops.rope_table(ctx.positions, self.inv_freq_v)
         ops.pooled_attention(qkv, kv, pooled, ctx, out, nh, self.scale, self.size, self.pool,
-                             self.inv_freq_v if self.rotate_values else None)
+                             self.inv_freq_v if self.rotate_values else None, turn_back)
         return linear.linear(out, self.w_o)
 
 

@@ -5,11 +5,15 @@
 ``token_side``: every layer owns a slice of ``dim`` entries of a second, narrow embedding table (``table_name``
 [vocab, parts * dim], shared by the layers; layer ``part`` reads [part dim, (part + 1) dim)).  With c that slice of the
 token's row:  y = proj (gelu_tanh(gate x) o c);  x <- x + y / sqrt(mean y^2 + eps) o norm, an RMS norm with a plain
-weight whatever norm the model uses elsewhere.  One kernel per layer, which also takes the sum that is still due.
+weight whatever norm the model uses elsewhere.  Both maps are matrix products like any other (the first reads the
+stream itself: the kernel that takes the sum still due also leaves its rows rounded to the products' type); the gate
+between them is float; the norm of y and the sum into x are one kernel.
 """
 from __future__ import annotations
 
-from ..kernels import ops
+import torch
+
+from ..kernels import linear, ops
 from ..weights.spec import TensorSpec
 from .base import Scale, TokenInput, register_part
 
@@ -42,10 +46,20 @@ class TokenSide(TokenInput):
 
     def load(self, get, rt):
         self.rt = rt
-        self.table, self.gate, self.proj, self.weight = (get(s) for s in self.tensor_specs())
+        self.table, gate, proj, self.weight = (get(s) for s in self.tensor_specs())
+        self.gate, self.proj = linear.prepare_weight(gate), linear.prepare_weight(proj)
 
     def forward(self, x, ctx, delta=None, delta_scale=None):
-        ops.token_side(x, ctx.token_ids, self.table, self.part, self.gate, self.proj, self.weight, self.eps, delta, delta_scale)
+        N = x.shape[0]
+        if self.rt.dtype == torch.float32:
+            if delta is not None:
+                ops.layer_norm(x, None, 0.0, None, delta=delta, delta_scale=delta_scale)
+            rows = x
+        else:
+            rows = ops.layer_norm(x, None, 0.0, self.rt.empty(N, self.hidden_size), delta=delta, delta_scale=delta_scale)
+        z = linear.linear(rows, self.gate)
+        g = ops.side_gate(z, ctx.token_ids, self.table, self.part, self.rt.empty(N, self.dim))
+        ops.rms_norm_add(linear.linear(g, self.proj), self.weight, self.eps, x)
 
 
 register_part("scale", "layer_scale", LayerScale)

@@ -64,10 +64,15 @@ SHAPES = {
         gru_layer(33, dense(72, 0.5)),
         attention_layer(6, 3, 16, 16, 0.3, 50, 7, 10000.0, 16, None)]),
 }
-PAGES = {"P": 16, "Q": 8, "R": 4}
+# heads of 64 and of 32 with values of the same size and pages of 16: in bfloat16 these attentions run on the matrix cores
+SHAPES["S"] = config(257, 160, 1e-5, 16, [
+    attention_layer(6, 2, 64, 64, 0.11, 40, 12, 10000.0, 32, moe(64, 6, 2)),
+    gru_layer(192, dense(192, 1.5)),
+    attention_layer(4, 4, 32, 32, 0.18, 16, 16, 10000.0, 32, dense(128, 3.0))], loop=(0, 1, 2))
+PAGES = {"P": 16, "Q": 8, "R": 4, "S": 16}
 # seeds of the shapes' weights: a router's choice is a comparison of floats, and with some weights a token's last chosen
 # and first unchosen expert lie closer together than bfloat16 activations can tell apart
-SEEDS = {"P": 84, "Q": 94, "R": 81}
+SEEDS = {"P": 84, "Q": 92, "R": 81, "S": 98}
 
 
 def tensor_shapes(cfg):
@@ -126,10 +131,10 @@ def random_weights(cfg, seed, dtype=torch.bfloat16):
             # the side input is normalised after its gate: where every gate of a token is shut, what is left of it is
             # rounding blown up to full size.  Gates of order one keep some of them open
             t = r * (0.03 / math.sqrt(shape[-1]))
-        elif leaf == "down" and ".mlp.e" in name:
+        elif ".mlp.e" in name:
             # a token whose two best experts tie may run another expert in bfloat16 than in 64-bit; small experts keep
             # what such a token does to the logits within the bound that rounding sets (32-bit sees them exactly)
-            t = r * (0.4 / math.sqrt(shape[-1]))
+            t = r * ((0.3 if leaf == "down" else 1.0) / math.sqrt(shape[-1]))
         else:
             t = r * (2.0 / math.sqrt(shape[-1]))
         w[name] = t.to(dtype).contiguous()
@@ -317,27 +322,34 @@ def test_layer_norm_sums_and_rows(dtype, H):
 
 @gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,d,parts", [(96, 8, 4), (130, 5, 3), (512, 1, 2), (64, 33, 1)])
-def test_token_side_input(dtype, H, d, parts):
-    from llm_infrence_engine_amd.kernels import ops
+@pytest.mark.parametrize("H,d,parts,N", [(96, 8, 4, 11), (130, 5, 3, 11), (512, 1, 2, 3), (64, 33, 1, 11), (256, 64, 2, 200)])
+def test_token_side_input(dtype, H, d, parts, N):
+    """Every layer's slice of the narrow table, with the scaled sum that is still due riding along."""
+    from llm_infrence_engine_amd.parts.base import Runtime
+    from llm_infrence_engine_amd.parts.side import TokenSide
 
     g = torch.Generator().manual_seed(H + d)
-    N, V = 11, 50
+    V = 50
     x = 2.0 * torch.randn(N, H, generator=g)
     y = torch.randn(N, H, generator=g).to(dtype)
     s = 0.5 + torch.rand(H, generator=g)
-    table = torch.randn(V, parts * d, generator=g).to(dtype)
-    gate = (torch.randn(d, H, generator=g) / math.sqrt(H)).to(dtype)
-    proj = torch.randn(H, d, generator=g).to(dtype)
-    wn = 1.0 + 0.2 * torch.randn(H, generator=g)
+    w = {"side.embed": torch.randn(V, parts * d, generator=g).to(dtype), "p.gate": (0.3 * torch.randn(d, H, generator=g) / math.sqrt(H)).to(dtype),
+         "p.proj": torch.randn(H, d, generator=g).to(dtype), "p.norm": 1.0 + 0.2 * torch.randn(H, generator=g)}
     ids = torch.randint(0, V, (N,), generator=g)
+    ctx = _Ctx([N], [0])
+    ctx.token_ids = ids.int().cuda()
     for part in range(parts):
         total = x.double() + s.double() * y.double()
-        w = {"side.embed": table.double(), "p.gate": gate.double(), "p.proj": proj.double(), "p.norm": wn.double()}
-        want = total + P.side_input(total, ids, part, w, "p.", d, 1e-6)
+        want = total + P.side_input(total, ids, part, {k_: v_.double() for k_, v_ in w.items()}, "p.", d, 1e-6)
+        side = TokenSide("p.", H, V, d, part, parts, 1e-6)
+        side.load(lambda spec: (w[spec.name].float() if spec.role == "norm" else w[spec.name].to(dtype)).cuda(), Runtime(torch.device("cuda"), dtype))
         xd = x.cuda()
-        ops.token_side(xd, ids.int().cuda(), table.cuda(), part, gate.cuda(), proj.cuda(), wn.cuda(), 1e-6, y.cuda(), s.cuda())
-        assert (xd.cpu().double() - want).abs().max() < 2e-5 * max(1.0, float(want.abs().max()))
+        side.forward(xd, ctx, delta=y.cuda(), delta_scale=s.cuda())
+        assert (xd.cpu().double() - want).abs().max() < (2e-5 if dtype == torch.float32 else 3e-2) * max(1.0, float(want.abs().max()))
+        xd = x.cuda()
+        side.forward(xd, ctx)                  # nothing due
+        want = x.double() + P.side_input(x.double(), ids, part, {k_: v_.double() for k_, v_ in w.items()}, "p.", d, 1e-6)
+        assert (xd.cpu().double() - want).abs().max() < (2e-5 if dtype == torch.float32 else 3e-2) * max(1.0, float(want.abs().max()))
 
 
 @gpu
@@ -373,8 +385,8 @@ def test_mingru_in_portions_and_batches(dtype, C):
 
 
 class _KV:
-    def __init__(self, k, v, table, rows, slots, stride=1, store=True):
-        self.pages, self.transposed = {"k": k, "v": v}, {"k": False, "v": False}
+    def __init__(self, k, v, table, rows, slots, stride=1, store=True, flipped=False):
+        self.pages, self.transposed = {"k": k, "v": v}, {"k": False, "v": flipped}
         self.block_table, self.table_rows, self.slot_mapping, self.store, self.stride = table, rows, slots, store, stride
 
 
@@ -416,12 +428,24 @@ def test_window_and_pooled_blocks_through_the_pages(dtype, H, G, D, E, page, siz
     want = P.windowed_pooled_attention(qt.to(dtype).double(), kt.repeat_interleave(rep, 1), vt.repeat_interleave(rep, 1), scale, size, pool,
                                        k_mean.repeat_interleave(rep, 1), v_mean.repeat_interleave(rep, 1))
     want = P.turn_pairs(want, pos, base, E, sign=-1.0)[T - Tq:]
+    # keys made loud after the turn cannot come from a projection: write the turned keys back through the inverse turn
+    k_src = P.turn_pairs(kt, pos, base, dims, sign=-1.0)
     # pages in no order for tokens and for blocks; the kernels store
     n_pages, n_bpages = -(-T // page), -(-max(nb, 1) // page)
     order = [int(x) for x in np.random.default_rng(1).permutation(np.arange(1, 1 + n_pages))]
     border = [int(x) for x in np.random.default_rng(2).permutation(np.arange(1, 1 + n_bpages))]
-    k_pages, v_pages, table = _paged(torch.zeros(T, G, D), torch.zeros(T, G, E), page, order, dtype)
-    pk_pages, pv_pages, ptable = _paged(torch.zeros(max(nb, 1), G, D), torch.zeros(max(nb, 1), G, E), page, border, dtype)
+    for flipped in (False, True):
+        _through_the_pages(dtype, H, G, D, E, page, size, pool, dims, T, Tq, base, q, k_src, v, scale, want, order, border, nb, flipped,
+                           blind_check=(j_in, i1, qt, kt, vt, rep, pos))
+
+
+def _through_the_pages(dtype, H, G, D, E, page, size, pool, dims, T, Tq, base, q, k_src, v, scale, want, order, border, nb, flipped,
+                       blind_check):
+    from llm_infrence_engine_amd.kernels import ops
+
+    j_in, i1, qt, kt, vt, rep, pos = blind_check
+    k_pages, v_pages, table = _paged(torch.zeros(T, G, D), torch.zeros(T, G, E), page, order, dtype, flipped)
+    pk_pages, pv_pages, ptable = _paged(torch.zeros(max(nb, 1), G, D), torch.zeros(max(nb, 1), G, E), page, border, dtype, flipped)
     k_pages.fill_(50.0), v_pages.fill_(50.0), pk_pages.fill_(50.0), pv_pages.fill_(50.0)
     if ptable.shape[1] < table.shape[1]:
         ptable = torch.cat([ptable, torch.zeros(2, table.shape[1] - ptable.shape[1], dtype=torch.int32, device="cuda")], 1)
@@ -430,9 +454,8 @@ def test_window_and_pooled_blocks_through_the_pages(dtype, H, G, D, E, page, siz
     rows = torch.tensor([1], dtype=torch.int32, device="cuda")
     f = lambda n, th: (th ** (-torch.arange(0, n, 2, dtype=torch.float64) / max(1, n))).float().cuda()
     inv_freq, inv_freq_v = f(dims, base), f(E, base)
-    # keys made loud after the turn cannot come from a projection: write the turned keys back through the inverse turn
-    k_src = P.turn_pairs(kt, pos, base, dims, sign=-1.0)
     outs = []
+    on_cores = (flipped and dtype == torch.bfloat16 and D == E and ops.attention_mfma_supported(D, page))
     for a, b in ((0, 101), (101, T - Tq), (T - Tq, T)):
         n = b - a
         ctx = _Ctx([n], [0], [a])
@@ -441,15 +464,32 @@ def test_window_and_pooled_blocks_through_the_pages(dtype, H, G, D, E, page, siz
         bslots = torch.tensor([border[((int(t) + 1) // pool - 1) // page] * page + ((int(t) + 1) // pool - 1) % page
                                if (int(t) + 1) % pool == 0 else -1 for t in p_], dtype=torch.int32, device="cuda")
         qkv = torch.cat([q[a:b].reshape(n, H * D).double(), k_src[a:b].reshape(n, G * D), v[a:b].reshape(n, G * E).double()], 1).to(dtype).cuda()
-        kv, pooled = _KV(k_pages, v_pages, table, rows, slots), _KV(pk_pages, pv_pages, ptable, rows, bslots, pool)
+        kv = _KV(k_pages, v_pages, table, rows, slots, flipped=flipped)
+        pooled = _KV(pk_pages, pv_pages, ptable, rows, bslots, pool, flipped=flipped)
         ops.pairs_rotate_store(qkv, H, G, D, E, dims, ctx.positions, inv_freq, inv_freq_v, kv)
         ops.pool_store(kv, pooled, ctx, pool)
         out = torch.empty(n, H * E, dtype=dtype, device="cuda")
-        ops.pooled_attention(qkv, kv, pooled, ctx, out, H, scale, size, pool, inv_freq_v)
+        ops.pooled_attention(qkv, kv, pooled, ctx, out, H, scale, size, pool, inv_freq_v, matrix_cores=True if on_cores else None)
         outs.append(out.cpu())
+        if on_cores:      # the same step on the vector ALUs
+            again = torch.empty(n, H * E, dtype=dtype, device="cuda")
+            ops.pooled_attention(qkv, kv, pooled, ctx, again, H, scale, size, pool, inv_freq_v, matrix_cores=False)
+            assert (again.float() - out.float()).abs().max() < 6e-2
     err = (outs[-1].double().reshape(Tq, H, E) - want).abs().max()
-    assert err < (1e-4 if dtype == torch.float32 else 6e-2), float(err)
-    if dtype == torch.float32:          # what the loud keys are there for
+    assert err < (1e-4 if dtype == torch.float32 else 6e-2), (flipped, float(err))
+    if on_cores:
+        # single tokens after it, two requests' worth of columns in one step: the narrow tiles of a decode step
+        for t in (T - 3, T - 1):
+            ctx = _Ctx([1], [0], [t])
+            qkv = torch.cat([q[t:t + 1].reshape(1, H * D).double(), k_src[t:t + 1].reshape(1, G * D), v[t:t + 1].reshape(1, G * E).double()], 1).to(dtype).cuda()
+            kv = _KV(k_pages, v_pages, table, rows, None, flipped=flipped, store=False)
+            pooled = _KV(pk_pages, pv_pages, ptable, rows, None, pool, flipped=flipped, store=False)
+            ops.pairs_rotate_store(qkv, H, G, D, E, dims, ctx.positions, inv_freq, inv_freq_v, kv)
+            out = torch.empty(1, H * E, dtype=dtype, device="cuda")
+            ops.pooled_attention(qkv, kv, pooled, ctx, out, H, scale, size, pool, inv_freq_v, matrix_cores=True)
+            err = (out.cpu().double().reshape(H, E) - want[t - (T - Tq)]).abs().max()
+            assert err < 6e-2, (t, float(err))
+    if dtype == torch.float32 and not flipped:          # what the loud keys are there for
         blind = P.windowed_pooled_attention(qt, kt.repeat_interleave(rep, 1), vt.repeat_interleave(rep, 1), scale, max(1, size - 1), pool)
         if j_in >= 0 and size > 1:
             assert (P.turn_pairs(blind, pos, base, E, sign=-1.0)[i1] - want[i1 - (T - Tq)]).abs().max() > 0.05
@@ -525,7 +565,8 @@ def shape(request, tmp_path_factory):
     cfg = SHAPES[name]
     weights = random_weights(cfg, seed=SEEDS[name])
     folder = write_model(tmp_path_factory.mktemp("kuvazen" + name), cfg, weights)
-    lengths = {"P": [5, 61, 2, 130, 33, 48], "Q": [1, 9, 90, 47, 110, 64], "R": [3, 26, 70, 17, 2, 41, 60, 33]}[name]
+    lengths = {"P": [5, 61, 2, 130, 33, 48], "Q": [1, 9, 90, 47, 110, 64], "R": [3, 26, 70, 17, 2, 41, 60, 33],
+               "S": [70, 3, 140, 50, 97, 33]}[name]
     reqs = requests_for(cfg["vocab"], lengths, seed=ord(name))
     w64 = {k: v.double() for k, v in weights.items()}
     want, noise = {}, {}
