@@ -114,22 +114,7 @@ __device__ __forceinline__ void load_values(ValueBlock<CT>& b, const bf16* __res
 // but only D / VS of the output's dims, so it reads all keys and 1 / VS of the values.  A compute unit draws
 // its data at a small fraction of the chip's rate, so when a step has fewer tiles than the chip has units this
 // shortens the longest chain without a second kernel; the blocks write disjoint dims and share nothing.
-//
-// POOL (general shape, with a window): beside the window's tokens a column sees one pooled key and value for every
-// whole block of `pool` tokens that lies before its window: entries 0 .. (pos - window + 1) / pool - 1 of a second set
-// of pages (pk_pages, pvt_pages, through pool_table: entry b at index b).  The pooled entries are walked first, as
-// blocks of 32 like any others and by the same waves in turn; only where a block's keys come from and which of them a
-// column sees differ.  turn_back (may be null): float2 [tokens, D / 2], the cosine and sine of an angle per token and pair
-// of neighbouring entries; the result's entries 2m, 2m + 1 are turned by minus that angle before they are stored.
-struct PoolArgs {
-  const bf16* pk_pages;
-  const bf16* pvt_pages;
-  const int* pool_table;
-  const float2* turn_back;
-  int pool;
-};
-
-template <int D, int NT, int WAVES, bool SPLIT, int VS, bool SINK, bool POOL = false>
+template <int D, int NT, int WAVES, bool SPLIT, int VS, bool SINK>
 __global__ void __launch_bounds__(WAVES * MS_WAVE, (NT > 1 ? 2 : 1))
 attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* __restrict__ k_pages,
                       const bf16* __restrict__ vt_pages, const int* __restrict__ block_table, int table_stride,
@@ -137,8 +122,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
                       const int* __restrict__ context_lens, bf16* __restrict__ out, size_t out_stride,
                       float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv, int page_size,
                       int page_shift, float scale_log2e, int window, int min_blocks, int n_splits,
-                      const float* __restrict__ sink, PoolArgs pa = PoolArgs{}) {
-  static_assert(!POOL || (!SPLIT && !SINK), "pooled blocks come with the general shape and without a sink");
+                      const float* __restrict__ sink) {
   // SPLIT: min_blocks and n_splits say how a request's key blocks are spread.  Else min_blocks != 0 asks for
   // the order of tiles in which a long tile's companion on its CU is a short one (see below), and n_splits is
   // the number of requests whose tiles the grid's second dimension runs over (0: one tile to a request)
@@ -200,7 +184,6 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   }
   const int row = table_rows ? table_rows[r] : r;
   const int* table = block_table + (size_t)row * table_stride;
-  const int* ptable = POOL ? pa.pool_table + (size_t)row * table_stride : nullptr;
   // Without a window a wave's first key block is known before the request's lengths are: ask for its page
   // ids at once, so that they travel together with the lengths instead of after them.
   int first_pages[2] = {0, 0};
@@ -241,15 +224,6 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
     blk_end = min(blk_end, blk_begin + per);
     if (blk_begin >= blk_end) return;
   }
-
-  // POOL: the pooled entries that the tile's last column sees come first, as the blocks vfirst .. blk_begin - 1
-  const auto seen_blocks = [&](int p) { return POOL && p - window + 1 >= pa.pool ? (p - window + 1) / pa.pool : 0; };
-  const int pool_hi = seen_blocks(key_hi) - 1;                 // the last pooled entry any column of the tile sees
-  const int vfirst = blk_begin - (pool_hi + 32) / 32;          // (pool_hi = -1: no such block)
-  const int pool_all = seen_blocks(first_pos);                 // entries below this one are seen by every column
-  // where the keys of block blk come from: (first entry, last entry that may be read, pooled or not)
-  const auto is_pooled = [&](int blk) { return POOL && blk < blk_begin; };
-  const auto base_of = [&](int blk) { return is_pooled(blk) ? (blk - vfirst) * 32 : blk * 32; };
 
   // this lane's columns
   int pos[NT];   // -1: an idle column (sees no key; its result is not written)
@@ -305,49 +279,39 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   KeyBlock<D> buf_k[2];
   ValueBlock<CT> buf_v[2];
   BlockPlace buf_at[2];
-  if (vfirst + wave < blk_end) {
+  if (blk_begin + wave < blk_end) {
     KeyBlock<D>& cur_k = buf_k[0];
     ValueBlock<CT>& cur_v = buf_v[0];
     BlockPlace& cur_at = buf_at[0];
-    const bool pooled = is_pooled(vfirst + wave);
-    const int base = base_of(vfirst + wave);
+    const int base = (blk_begin + wave) * 32;
     int pages[2];
     if (early) {  // blk_begin is 0 here; halves past the last key fall back to the null page
 #pragma unroll
       for (int u = 0; u < 2; ++u) pages[u] = base + u * 16 <= key_hi ? first_pages[u] : 0;
     } else {
-      pages_of(pooled ? ptable : table, base, pooled ? pool_hi : key_hi, pg, pages);
+      pages_of(table, base, key_hi, pg, pages);
     }
     cur_at = place_of(pages, base, g, nkv, pg, D);
-    load_keys<D>(cur_k, pooled ? pa.pk_pages : k_pages, cur_at, lane);
-    if (VALUES_EARLY) load_values<CT>(cur_v, pooled ? pa.pvt_pages : vt_pages, cur_at, pg, dim0, lane);
+    load_keys<D>(cur_k, k_pages, cur_at, lane);
+    if (VALUES_EARLY) load_values<CT>(cur_v, vt_pages, cur_at, pg, dim0, lane);
   }
   // The page ids of a block are asked for one block before its keys are: the keys' loads then go out at the top of
   // an iteration instead of behind a table lookup (8,192 tokens of the 0.5B shape: 235 -> 232 us; 2,048 tokens at
   // head size 128: 99.9 -> 96.7 us).  (Keeping the loads of two blocks in flight for narrow tiles was measured and
   // dropped: a decode tile's time is what its CU can draw, 102 KB at about 43 GB/s at 640 keys, not its waits.)
   int ahead_pages[2] = {0, 0};
-  if (vfirst + wave + WAVES < blk_end) {
-    const bool pooled = is_pooled(vfirst + wave + WAVES);
-    pages_of(pooled ? ptable : table, base_of(vfirst + wave + WAVES), pooled ? pool_hi : key_hi, pg, ahead_pages);
-  }
+  if (blk_begin + wave + WAVES < blk_end) pages_of(table, (blk_begin + wave + WAVES) * 32, key_hi, pg, ahead_pages);
   // One block of 32 keys: the step works on the buffers it is handed as current and fills those it is handed
   // as next; the loop below calls it with the two sets of buffers in turn, so nothing is copied between them.
   auto step = [&](int blk, KeyBlock<D>& cur_k, ValueBlock<CT>& cur_v, BlockPlace& cur_at, KeyBlock<D>& nxt_k,
                   ValueBlock<CT>& nxt_v, BlockPlace& nxt_at) __attribute__((always_inline)) {
-    const bool pooled = is_pooled(blk);
-    const int base = base_of(blk);
-    const int hi = pooled ? pool_hi : key_hi;      // the last entry of this block's source that may be read
-    if (!VALUES_EARLY) load_values<CT>(cur_v, pooled ? pa.pvt_pages : vt_pages, cur_at, pg, dim0, lane);
+    const int base = blk * 32;
+    if (!VALUES_EARLY) load_values<CT>(cur_v, vt_pages, cur_at, pg, dim0, lane);
     if (blk + WAVES < blk_end) {
-      const bool npooled = is_pooled(blk + WAVES);
-      nxt_at = place_of(ahead_pages, base_of(blk + WAVES), g, nkv, pg, D);
-      load_keys<D>(nxt_k, npooled ? pa.pk_pages : k_pages, nxt_at, lane);
-      if (VALUES_EARLY) load_values<CT>(nxt_v, npooled ? pa.pvt_pages : vt_pages, nxt_at, pg, dim0, lane);
-      if (blk + 2 * WAVES < blk_end) {
-        const bool apooled = is_pooled(blk + 2 * WAVES);
-        pages_of(apooled ? ptable : table, base_of(blk + 2 * WAVES), apooled ? pool_hi : key_hi, pg, ahead_pages);
-      }
+      nxt_at = place_of(ahead_pages, base + WAVES * 32, g, nkv, pg, D);
+      load_keys<D>(nxt_k, k_pages, nxt_at, lane);
+      if (VALUES_EARLY) load_values<CT>(nxt_v, vt_pages, nxt_at, pg, dim0, lane);
+      if (blk + 2 * WAVES < blk_end) pages_of(table, base + 2 * WAVES * 32, key_hi, pg, ahead_pages);
     }
 
     // scores: s[u][t] holds keys base + u*16 + kq*4 + (0..3) of column t*16 + col16
@@ -363,19 +327,18 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
       }
 
     // values past the last visible key may be anything a reused page still holds: make them zero
-    if (base + 31 > hi) {
+    if (base + 31 > key_hi) {
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (base + u * 16 + kq * 4 + i > hi) {
+          if (base + u * 16 + kq * 4 + i > key_hi) {
 #pragma unroll
             for (int c = 0; c < CT; ++c) cur_v.v[c][u][i] = (__bf16)0.0f;
           }
     }
 
-    const bool unmasked = pooled ? full_tile && base + 31 < pool_all
-                                 : full_tile && base + 31 <= first_pos && (window <= 0 || base > key_hi - window);
+    const bool unmasked = full_tile && base + 31 <= first_pos && (window <= 0 || base > key_hi - window);
     bf16x8 p[NT];
     float corr[NT], bmax[NT];
     bool moved = false;
@@ -400,8 +363,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const int key = base + u * 16 + kq * 4 + i;
-            const bool see = pooled ? key < seen_blocks(pos[t])
-                                    : key <= pos[t] && (window <= 0 || key > pos[t] - window);
+            const bool see = key <= pos[t] && (window <= 0 || key > pos[t] - window);
             const float v = see ? s[u][t][i] : -INFINITY;
             s[u][t][i] = v;
             bm = fmaxf(bm, v);
@@ -457,7 +419,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
       }
     }
   };
-  for (int blk = vfirst + wave; blk < blk_end; blk += 2 * WAVES) {
+  for (int blk = blk_begin + wave; blk < blk_end; blk += 2 * WAVES) {
     step(blk, buf_k[0], buf_v[0], buf_at[0], buf_k[1], buf_v[1], buf_at[1]);
     if (blk + WAVES < blk_end) step(blk + WAVES, buf_k[1], buf_v[1], buf_at[1], buf_k[0], buf_v[0], buf_at[0]);
   }
@@ -523,18 +485,8 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
 #pragma unroll
       for (int c = 0; c < CT; ++c) {
         bf16x4 w;
-        if (POOL && pa.turn_back) {     // a lane's four dims are two pairs of neighbours
 #pragma unroll
-          for (int i = 0; i < 4; i += 2) {
-            const float2 cs = pa.turn_back[(size_t)tok * (D / 2) + ((dim0 + c * 16 + kq * 4 + i) >> 1)];
-            const float a = o[c][t][i] * inv, b = o[c][t][i + 1] * inv;
-            w[i] = (__bf16)(a * cs.x + b * cs.y);
-            w[i + 1] = (__bf16)(b * cs.x - a * cs.y);
-          }
-        } else {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) w[i] = (__bf16)(o[c][t][i] * inv);
-        }
+        for (int i = 0; i < 4; ++i) w[i] = (__bf16)(o[c][t][i] * inv);
         *reinterpret_cast<bf16x4*>(op + c * 16) = w;
       }
     }
@@ -616,22 +568,6 @@ int launch_general(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt
     return ms_launch_status();
   }
   attention_mfma_kernel<D, NT, WAVES, false, VS, false><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, table_rows, q_start, ctx, out, out_stride, nullptr, nullptr, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, pair_order, scan, nullptr);
-  return ms_launch_status();
-}
-
-template <int D, int NT, int WAVES, int VS>
-int launch_pooled(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, const int* table, int table_stride,
-                  const int* table_rows, const int* q_start, const int* ctx, bf16* out, size_t out_stride,
-                  int n_requests, int n_tokens, int max_q_len, int nh, int nkv, int page_size, float scale,
-                  int window, PoolArgs pa, hipStream_t stream) {
-  const int rep = nh / nkv;
-  const long long per_request = ((long long)max_q_len * rep + 16 * NT - 1) / (16 * NT);
-  long long tiles = (long long)n_tokens * rep / (16 * NT) + n_requests;
-  if (tiles > per_request * n_requests) tiles = per_request * n_requests;
-  if (tiles > 65535) return MS_UNSUPPORTED;   // grid.y
-  const int scan = per_request == 1 ? 0 : n_requests;
-  dim3 grid(nkv, (unsigned)tiles, VS), block(WAVES * MS_WAVE);
-  attention_mfma_kernel<D, NT, WAVES, false, VS, false, true><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, table_rows, q_start, ctx, out, out_stride, nullptr, nullptr, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, 0, scan, nullptr, pa);
   return ms_launch_status();
 }
 
@@ -745,38 +681,5 @@ extern "C" int ms_paged_attention_mfma_decode(const void* q, long long q_stride,
   if (head_dim == 32) GO(32);
   if (head_dim == 64) GO(64);
   GO(128);
-#undef GO
-}
-
-// A window of `window` tokens and pooled blocks of `pool` tokens before it (see POOL above).  As ms_paged_attention_mfma,
-// plus pk_pages [P2, nkv, page_size, d], pvt_pages [P2, nkv, d, page_size] (entry b of a request at index b of its row of
-// pool_table, int32 [rows, table_stride]) and turn_back (may be null) float [n_tokens, d / 2, 2], (cos, sin) per token and pair.
-extern "C" int ms_pooled_attention_mfma(const void* q, long long q_stride, const void* k_pages, const void* vt_pages,
-                                        const int* block_table, const void* pk_pages, const void* pvt_pages,
-                                        const int* pool_table, int table_stride, const int* table_rows,
-                                        const int* q_start, const int* context_lens, const float* turn_back, void* out,
-                                        long long out_stride, int n_requests, int n_tokens, int max_q_len, int num_heads,
-                                        int num_kv_heads, int head_dim, int page_size, float scale, int window, int pool,
-                                        hipStream_t stream) {
-  if (n_requests <= 0 || max_q_len <= 0 || n_tokens <= 0) return MS_OK;
-  if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || table_stride <= 0 || window <= 0 || pool <= 0 ||
-      pk_pages == nullptr || pvt_pages == nullptr || pool_table == nullptr)
-    return MS_BAD_ARG;
-  if (!(scale > 0.f)) return MS_BAD_ARG;
-  if (!ms_attention_mfma_supported(head_dim, page_size)) return MS_UNSUPPORTED;
-  if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q % 16) || ((uintptr_t)out % 8)) return MS_UNSUPPORTED;
-  if (n_requests > 65535 || num_kv_heads > 65535) return MS_UNSUPPORTED;
-  if ((uintptr_t)turn_back % 8) return MS_BAD_ARG;
-  const PoolArgs pa = {(const bf16*)pk_pages, (const bf16*)pvt_pages, pool_table, (const float2*)turn_back, pool};
-#define GO(D, NT, WV) return launch_pooled<D, NT, WV, 1>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, table_rows, q_start, context_lens, (bf16*)out, out_stride, n_requests, n_tokens, max_q_len, num_heads, num_kv_heads, page_size, scale, window, pa, stream)
-  const int cols = max_q_len * (num_heads / num_kv_heads);
-  if (cols > 16) {
-    if (head_dim == 32) GO(32, 2, 4);
-    if (head_dim == 64) GO(64, 2, 4);
-    GO(128, 2, 4);
-  }
-  if (head_dim == 32) GO(32, 1, 8);
-  if (head_dim == 64) GO(64, 1, 8);
-  GO(128, 1, 8);
 #undef GO
 }
