@@ -394,7 +394,7 @@ class _KV:
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,D,E,page,size,pool,dims", [
     (6, 2, 16, 24, 4, 20, 5, 8), (4, 1, 64, 64, 16, 96, 12, 64), (3, 3, 32, 8, 8, 7, 16, 0), (2, 1, 6, 10, 4, 1, 1, 6),
-    (2, 2, 48, 64, 16, 33, 3, 32), (8, 2, 128, 128, 16, 16, 16, 64)])
+    (2, 2, 40, 56, 16, 33, 3, 32), (8, 2, 128, 128, 16, 16, 16, 64)])
 def test_window_and_pooled_blocks_through_the_pages(dtype, H, G, D, E, page, size, pool, dims):
     """One sequence of 230 tokens stored in three steps (the cuts fall inside a page, a block and the window) into pages
     in no order, then the last 60 queries.  For one query the key just inside the window and, for another, every key of
