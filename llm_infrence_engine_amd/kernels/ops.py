@@ -1549,7 +1549,7 @@ def pooled_attention(q: torch.Tensor, kv, pooled, ctx, out: torch.Tensor, num_he
         _check(inv_freq_v, "inv_freq_v", torch.float32, (dv // 2,))
     _check(ctx.token_req, "token_req", torch.int32, (N,))
     _check(ctx.positions, "positions", torch.int32, (N,))
-    can = (q.dtype == torch.bfloat16 and flipped and dv == d and pool > 0 and attention_mfma_supported(d, page_size)
+    can = (q.dtype == torch.bfloat16 and flipped and dv == d and pool > 0 and scale > 0 and attention_mfma_supported(d, page_size)
            and q.data_ptr() % 16 == 0 and (N == 1 or q.stride(0) % 8 == 0))
     if matrix_cores and not can:
         raise UnsupportedShape("the matrix-core kernel takes bfloat16, transposed value pages of the keys' size (32, 64 or "

@@ -69,10 +69,14 @@ SHAPES["S"] = config(257, 160, 1e-5, 16, [
     attention_layer(6, 2, 64, 64, 0.11, 40, 12, 10000.0, 32, moe(64, 6, 2)),
     gru_layer(192, dense(192, 1.5)),
     attention_layer(4, 4, 32, 32, 0.18, 16, 16, 10000.0, 32, dense(128, 3.0))], loop=(0, 1, 2))
-PAGES = {"P": 16, "Q": 8, "R": 4, "S": 16}
+# sizes that are multiples of nothing much (a width of 100, heads of 10 and 14, five of them), the whole model one looped stretch
+SHAPES["T"] = config(77, 100, 1e-5, 3, [
+    gru_layer(50, moe(20, 3, 1)),
+    attention_layer(5, 5, 10, 14, 0.3, 9, 4, 10000.0, 6, dense(36, 1.2))], loop=(0, 2, 2))
+PAGES = {"P": 16, "Q": 8, "R": 4, "S": 16, "T": 16}
 # seeds of the shapes' weights: a router's choice is a comparison of floats, and with some weights a token's last chosen
 # and first unchosen expert lie closer together than bfloat16 activations can tell apart
-SEEDS = {"P": 84, "Q": 92, "R": 81, "S": 98}
+SEEDS = {"P": 84, "Q": 92, "R": 81, "S": 98, "T": 82}
 
 
 def tensor_shapes(cfg):
@@ -394,7 +398,8 @@ class _KV:
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,D,E,page,size,pool,dims", [
     (6, 2, 16, 24, 4, 20, 5, 8), (4, 1, 64, 64, 16, 96, 12, 64), (3, 3, 32, 8, 8, 7, 16, 0), (2, 1, 6, 10, 4, 1, 1, 6),
-    (2, 2, 40, 56, 16, 33, 3, 32), (8, 2, 128, 128, 16, 16, 16, 64)])
+    (2, 2, 40, 56, 16, 33, 3, 32), (8, 2, 128, 128, 16, 16, 16, 64), (4, 2, 32, 32, 16, 1, 1, 32), (2, 1, 64, 64, 16, 5, 3, 0),
+    (3, 1, 48, 48, 16, 70, 9, 48)])
 def test_window_and_pooled_blocks_through_the_pages(dtype, H, G, D, E, page, size, pool, dims):
     """One sequence of 230 tokens stored in three steps (the cuts fall inside a page, a block and the window) into pages
     in no order, then the last 60 queries.  For one query the key just inside the window and, for another, every key of
@@ -566,7 +571,7 @@ def shape(request, tmp_path_factory):
     weights = random_weights(cfg, seed=SEEDS[name])
     folder = write_model(tmp_path_factory.mktemp("kuvazen" + name), cfg, weights)
     lengths = {"P": [5, 61, 2, 130, 33, 48], "Q": [1, 9, 90, 47, 110, 64], "R": [3, 26, 70, 17, 2, 41, 60, 33],
-               "S": [70, 3, 140, 50, 97, 33]}[name]
+               "S": [70, 3, 140, 50, 97, 33], "T": [40, 2, 90, 17, 66]}[name]
     reqs = requests_for(cfg["vocab"], lengths, seed=ord(name))
     w64 = {k: v.double() for k, v in weights.items()}
     want, noise = {}, {}
