@@ -264,9 +264,10 @@ int ms_layer_norm(float* x, const void* delta, int delta_dtype, const float* dsc
 int ms_side_gate(const void* z, long long z_stride, const int* token_ids, const void* table, long long table_stride, int part,
                  void* out, int n_tokens, int d, int dtype, hipStream_t stream);
 // ---- minGRU (csrc/mingru.hip)
+int ms_mingru_chunk();
 int ms_mingru_scan(const void* zxg, long long in_stride, const float* bz, const float* bx, float* state, const int* q_start,
-                   const int* state_slots, void* out, long long out_stride, int n_requests, int C, int long_portions,
-                   int dtype, hipStream_t stream);
+                   const int* state_slots, void* out, long long out_stride, int n_requests, int C, int max_q_len,
+                   float* scratch, int dtype, hipStream_t stream);
 // ---- window + pooled blocks attention (csrc/pooled_attention.hip)
 int ms_pairs_rotate_store(void* qkv, long long stride, const int* positions, const float* inv_freq, const float* inv_freq_v,
                           const int* slots, void* k_pages, void* v_pages, int n_tokens, int num_heads, int num_kv_heads,

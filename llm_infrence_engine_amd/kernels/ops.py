@@ -103,8 +103,9 @@ _SIGNATURES = {
     "ms_moe_route": [_c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "ms_layer_norm": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "ms_side_gate": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
-    "ms_mingru_scan": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int,
-                       _c_ptr],
+    "ms_mingru_chunk": [],
+    "ms_mingru_scan": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_ptr,
+                       _c_int, _c_ptr],
     "ms_pairs_rotate_store": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
                               _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_pool_store": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
@@ -1438,7 +1439,7 @@ def mingru_scan(zxg: torch.Tensor, bias_z: Optional[torch.Tensor], bias_x: Optio
                 ctx, out: torch.Tensor) -> torch.Tensor:
     """The minGRU recurrence over the step's portions, from and into ``state`` float [slots, C]: with the thirds pz | px | pg
     of a row of zxg [N, 3C]: z = sigmoid(pz + bias_z); u = px + bias_x; c = u + 1/2 (u >= 0) or sigmoid(u);
-    S <- (1 - z) S + z c; out = S * silu(pg)."""
+    S <- (1 - z) S + z c; out = S * silu(pg).  ``ctx.max_q_len`` bounds the portions' lengths."""
     C = state.shape[1]
     stride = _rows2d(zxg, "zxg", None, 3 * C)
     N = zxg.shape[0]
@@ -1452,8 +1453,13 @@ def mingru_scan(zxg: torch.Tensor, bias_z: Optional[torch.Tensor], bias_x: Optio
     R = ctx.num_requests
     _check(ctx.q_start, "q_start", torch.int32, (R + 1,))
     _check(ctx.state_slots, "state_slots", torch.int32, (R,))
+    longest = max(1, int(ctx.max_q_len))
+    chunk = int(_get("ms_mingru_chunk")())
+    scratch = None
+    if longest > chunk:      # a long portion's chunks are spread over blocks; their pairs and starting states pass through here
+        scratch = torch.empty((R * (-(-longest // chunk)) * 2 + R) * C, dtype=torch.float32, device=zxg.device)
     _call("ms_mingru_scan", zxg.data_ptr(), stride, _ptr(bias_z), _ptr(bias_x), state.data_ptr(), ctx.q_start.data_ptr(),
-          ctx.state_slots.data_ptr(), out.data_ptr(), os_, R, C, int(ctx.max_q_len > 8), _code(zxg.dtype), _stream())
+          ctx.state_slots.data_ptr(), out.data_ptr(), os_, R, C, longest, _ptr(scratch), _code(zxg.dtype), _stream())
     return out
 
 
@@ -1562,12 +1568,16 @@ def pooled_attention(q: torch.Tensor, kv, pooled, ctx, out: torch.Tensor, num_he
             turn_back = rope_table(ctx.positions, inv_freq_v)
         if turn_back is not None:
             _check(turn_back, "turn_back", torch.float32, (N, d // 2, 2))
-        _call("ms_pooled_attention_mfma", q.data_ptr(), q.stride(0) if N > 1 else q.shape[1], k.data_ptr(), v.data_ptr(),
-              kv.block_table.data_ptr(), pk.data_ptr(), pv.data_ptr(), ptab.data_ptr(), kv.block_table.shape[1],
-              _ptr(kv.table_rows), ctx.q_start.data_ptr(), ctx.context_lens.data_ptr(), _ptr(turn_back), out.data_ptr(),
-              num_heads * dv, R, N, max(1, ctx.max_q_len), num_heads, nkv, d, page_size, float(scale), int(size), int(pool),
-              _stream())
-        return out
+        try:
+            _call("ms_pooled_attention_mfma", q.data_ptr(), q.stride(0) if N > 1 else q.shape[1], k.data_ptr(), v.data_ptr(),
+                  kv.block_table.data_ptr(), pk.data_ptr(), pv.data_ptr(), ptab.data_ptr(), kv.block_table.shape[1],
+                  _ptr(kv.table_rows), ctx.q_start.data_ptr(), ctx.context_lens.data_ptr(), _ptr(turn_back), out.data_ptr(),
+                  num_heads * dv, R, N, max(1, ctx.max_q_len), num_heads, nkv, d, page_size, float(scale), int(size),
+                  int(pool), _stream())
+            return out
+        except UnsupportedShape:        # more tiles than a launch holds: the vector-ALU kernel takes any step
+            if matrix_cores:
+                raise
     _call("ms_pooled_attention", q.data_ptr(), q.stride(0) if N > 1 else q.shape[1], k.data_ptr(), v.data_ptr(),
           kv.block_table.data_ptr(), _ptr(pk), _ptr(pv), _ptr(ptab), kv.block_table.shape[1], _ptr(kv.table_rows),
           _ptr(ctx.n_live_tokens), ctx.token_req.data_ptr(), ctx.positions.data_ptr(), _ptr(inv_freq_v), out.data_ptr(),

@@ -680,6 +680,11 @@ def test_far_token_reaches_the_end(tmp_path, kind):
         _replay(folder, "float32", steps, tmp_path / mode, 2 * 448, 16)
         got = traces.collect(steps, tmp_path / mode, 97)
         assert np.abs(got[("a", 419)] - la).max() < 5e-4 and np.abs(got[("b", 419)] - lb).max() < 5e-4
+    # a model of one kind of layer alone (no state, or no pages at all) through the graphs of the bfloat16 path
+    steps = traces.bulk_then_single(reqs, tail=40)
+    _replay(folder, "bfloat16", steps, tmp_path / "bf16", 2 * 448, 16)
+    got = traces.collect(steps, tmp_path / "bf16", 97)
+    assert np.abs(got[("a", 419)] - la).max() < 0.15 and np.abs(got[("b", 419)] - lb).max() < 0.15
 
 
 @gpu
