@@ -6,8 +6,9 @@ from .qwen2 import Qwen2Config
 from .gemadra import GemadraConfig
 from .gidurax import GiduraxConfig
 from .kuvazen import KuvazenConfig
+from .silizen import SilizenConfig
 from .presets import PRESETS, preset
 
 __all__ = ["EngineConfig", "ConfigError", "build_spec", "config_class", "config_from_dict",
            "known_architectures", "load_config", "register_architecture", "LayerSpec", "ModelSpec",
-           "PartSpec", "Run", "layer", "Qwen2Config", "GemadraConfig", "GiduraxConfig", "KuvazenConfig", "PRESETS", "preset"]
+           "PartSpec", "Run", "layer", "Qwen2Config", "GemadraConfig", "GiduraxConfig", "KuvazenConfig", "SilizenConfig", "PRESETS", "preset"]

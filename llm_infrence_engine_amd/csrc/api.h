@@ -107,7 +107,8 @@ int ms_paged_attention_generic(const void* q, long long q_stride, const void* k_
                                const int* n_live_tokens, const int* token_req, const int* positions,
                                void* out, long long out_stride, int n_tokens, int num_heads, int num_kv_heads,
                                int head_dim, int value_dim, int page_size, long long num_pages, float scale, int window,
-                               int v_transposed, const float* sink, int dtype, hipStream_t stream);
+                               int v_transposed, const float* sink, float softcap, const float* slopes, const void* gate,
+                               long long gate_stride, float out_scale, int dtype, hipStream_t stream);
 
 int ms_attention_mfma_supported(int head_dim, int page_size);
 
@@ -173,9 +174,11 @@ int ms_gated_delta(const void* q, const void* k, const void* v, long long qkv_st
                    int single_tokens, int dtype, hipStream_t stream);
 
 // out[n, h, :] = o[n, h, :] / rms(o[n, h, :]) * weight * act(gate[n, h, :]), act the sigmoid or (gate_silu) z * sigmoid(z);
-// o float, gate and out in `dtype`.
+// o float, gate and out in `dtype`.  weight [vdim], shared by the heads, or with weight_per_head [heads * vdim]; `scale`
+// multiplies every result.
 int ms_gated_head_norm(const float* o, const float* weight, const void* gate, long long gate_stride, void* out,
-                       int n_tokens, int heads, int vdim, float eps, int gate_silu, int dtype, hipStream_t stream);
+                       int n_tokens, int heads, int vdim, float eps, int gate_silu, int weight_per_head, float scale,
+                       int dtype, hipStream_t stream);
 
 // xIELU with pq = (p, q) on the device.
 int ms_xielu(const void* x, const float* pq, void* out, long long total, int dtype, hipStream_t stream);
@@ -217,11 +220,12 @@ int ms_add_rows(float* x, const float* kept, const float* vec, int n_rows, int h
 
 // ---- heads normalised instead of rotated (csrc/qk_norm.hip): RMS norm of every q and k head with q_weight / k_weight
 // [head_dim] (null: no norm), q times 1 + coef * ln(floor((p + 1) / every) + 1) (coef 0: none), k and v stored into pages
-// (null: not stored); qkv [n, nh * head_dim + nkv * head_dim + nkv * value_dim]
+// (null: not stored); qkv [n, nh * head_dim + nkv * head_dim + nkv * value_dim].  unit_norm: the norm also without weights;
+// rot_dim > 0: after the norm, entry i and entry i + rot_dim / 2 of every q and k head turn by position * inv_freq[i]
 int ms_qk_norm_store(void* qkv, long long stride, const float* q_weight, const float* k_weight, float eps,
                      const int* positions, float coef, int every, const int* slots, void* k_pages, void* v_pages,
                      int n_tokens, int num_heads, int num_kv_heads, int head_dim, int value_dim, int page_size,
-                     int v_transposed, int dtype, hipStream_t stream);
+                     int v_transposed, int unit_norm, const float* inv_freq, int rot_dim, int dtype, hipStream_t stream);
 
 // ---- the selective scan of a state-space mixer (csrc/scan.hip)
 int ms_selective_scan(const void* x, long long x_stride, const float* dt_in, const float* dt_bias, const float* A,
@@ -259,7 +263,7 @@ int ms_moe_combine(const float* part, const int* ids, const float* weights, cons
                    int n_tokens, int top, int n_experts, int hidden, int dtype, hipStream_t stream);   // weights null: all 1
 
 // ---- layer norm and the gate of a token's side input (csrc/layer_norm.hip)
-int ms_layer_norm(float* x, const void* delta, int delta_dtype, const float* dscale, const float* w, const int* rows,
+int ms_layer_norm(float* x, const void* delta, int delta_dtype, const float* dscale, const float* w, const float* b, const int* rows,
                   void* out, int n_rows, int H, float eps, int write_back, int out_dtype, hipStream_t stream);
 int ms_side_gate(const void* z, long long z_stride, const int* token_ids, const void* table, long long table_stride, int part,
                  void* out, int n_tokens, int d, int dtype, hipStream_t stream);
@@ -295,5 +299,20 @@ int ms_clamped_glu(const void* gu, long long in_stride, void* out, long long out
                    float alpha, int dtype, hipStream_t stream);
 int ms_scaled_swiglu(const void* gu, long long in_stride, const float* factor, const int* row_item, void* out,
                      long long out_stride, int n_rows, int F, int dtype, hipStream_t stream);
+int ms_gelu_tanh_glu(const void* gu, long long in_stride, void* out, long long out_stride, int n_rows, int F, int dtype,
+                     hipStream_t stream);
+// ---- recurrences with a decay per key channel, the previous token's input, sums of two mixers (csrc/recurrence.hip)
+int ms_decay_recurrence(const void* q, const void* k, const void* v, long long q_stride, long long k_stride,
+                        long long v_stride, const float* z, const float* z_bias, int decay_kind, float inv_tau,
+                        const float* bonus, float q_scale, float* state, const int* q_start, const int* state_slots,
+                        float* out, int n_requests, int heads, int dim, int vdim, int dtype, hipStream_t stream);
+int ms_token_shift(const void* h, long long h_stride, const float* mu, void* state, const int* token_req,
+                   const int* q_start, const int* state_slots, const int* n_live_tokens, void* out, int n_tokens,
+                   int n_requests, int width, int n_mixes, int dtype, hipStream_t stream);
+int ms_pair_sum(const void* a, const void* b, float scale_a, float scale_b, const float* norm_a, const float* norm_b,
+                float eps, float* x, int n_rows, int width, int dtype, hipStream_t stream);
+int ms_tanh(void* x, long long total, int dtype, hipStream_t stream);
+int ms_concat_rows(const float* a, const float* b, void* out, int n_rows, int width_a, int width_b, int out_dtype,
+                   hipStream_t stream);
 
 }  // extern "C"

@@ -5,6 +5,9 @@
 // position, so what a reused page still holds from an earlier request cannot reach the result.
 // block_table int32 [rows, table_stride]; request r of the step has row table_rows[r] (null: row r).
 // n_live_tokens (null: all): a device int; tokens from that index on belong to no request and are skipped.
+// `softcap` > 0: a score s (already scaled) becomes softcap * tanh(s / softcap).  `slopes` (may be null): one number per
+// query head; slope * (distance of the key from the query) is taken off the score, after the cap.  `gate` (may be null):
+// one number per token and query head, the head's result is multiplied by sigmoid(gate); `out_scale` multiplies all.
 // This is the attention of the 32-bit path and the any-shape fallback of the bfloat16 path.
 #include "common.h"
 #include "api.h"
@@ -22,7 +25,8 @@ paged_attention_generic_kernel(const T* __restrict__ q, size_t q_stride, const T
                                const int* __restrict__ token_req, const int* __restrict__ positions,
                                T* __restrict__ out, size_t out_stride, int n_tokens, int nh, int nkv, int d, int dv,
                                int page_size, float scale, int window, int v_transposed,
-                               const float* __restrict__ sink) {
+                               const float* __restrict__ sink, float softcap, const float* __restrict__ slopes,
+                               const T* __restrict__ gate, size_t gate_stride, float out_scale) {
   __shared__ float qs[WAVES][MAX_D];
   const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
   const long long item = (long long)blockIdx.x * WAVES + wave;
@@ -43,6 +47,8 @@ paged_attention_generic_kernel(const T* __restrict__ q, size_t q_stride, const T
   int start = 0;
   if (window > 0 && pos - window + 1 > 0) start = pos - window + 1;
 
+  const float slope = slopes ? slopes[h] : 0.f;
+  const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
   float m = -INFINITY, l = 0.f;
   float acc[MAX_D / MS_WAVE];
 #pragma unroll
@@ -67,6 +73,8 @@ paged_attention_generic_kernel(const T* __restrict__ q, size_t q_stride, const T
       }
       for (; i < d; ++i) dot = fmaf(qs[wave][i], to_float(kp[i]), dot);
       s = dot;
+      if (softcap > 0.f) s = softcap * tanhf(s * inv_cap);
+      if (slopes) s -= slope * (float)(pos - j);
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -92,7 +100,8 @@ paged_attention_generic_kernel(const T* __restrict__ q, size_t q_stride, const T
   }
   T* op = out + (size_t)n * out_stride + (size_t)h * dv;
   if (sink) l += expf(sink[h] - m);   // m is finite: a token always sees its own key
-  const float inv = 1.0f / l;
+  float inv = out_scale / l;
+  if (gate) inv /= 1.0f + expf(-to_float(gate[(size_t)n * gate_stride + h]));
 #pragma unroll
   for (int c = 0; c < MAX_D / MS_WAVE; ++c) {
     const int i = lane + c * MS_WAVE;
@@ -108,7 +117,8 @@ extern "C" int ms_paged_attention_generic(const void* q, long long q_stride, con
                                           const int* positions, void* out, long long out_stride, int n_tokens,
                                           int num_heads, int num_kv_heads, int head_dim, int value_dim, int page_size,
                                           long long num_pages, float scale, int window, int v_transposed,
-                                          const float* sink, int dtype, hipStream_t stream) {
+                                          const float* sink, float softcap, const float* slopes, const void* gate,
+                                          long long gate_stride, float out_scale, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return MS_OK;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || page_size <= 0 || table_stride <= 0)
     return MS_BAD_ARG;
@@ -116,7 +126,7 @@ extern "C" int ms_paged_attention_generic(const void* q, long long q_stride, con
   if (num_pages * num_kv_heads * page_size >= (1ll << 31)) return MS_UNSUPPORTED;  // row index is an int
   const long long items = (long long)n_tokens * num_heads;
   dim3 grid((unsigned)((items + WAVES - 1) / WAVES)), block(WAVES * MS_WAVE);
-#define LAUNCH(T) paged_attention_generic_kernel<T><<<grid, block, 0, stream>>>((const T*)q, (size_t)q_stride, (const T*)k_pages, (const T*)v_pages, block_table, table_stride, table_rows, n_live_tokens, token_req, positions, (T*)out, (size_t)out_stride, n_tokens, num_heads, num_kv_heads, head_dim, value_dim, page_size, scale, window, v_transposed, sink)
+#define LAUNCH(T) paged_attention_generic_kernel<T><<<grid, block, 0, stream>>>((const T*)q, (size_t)q_stride, (const T*)k_pages, (const T*)v_pages, block_table, table_stride, table_rows, n_live_tokens, token_req, positions, (T*)out, (size_t)out_stride, n_tokens, num_heads, num_kv_heads, head_dim, value_dim, page_size, scale, window, v_transposed, sink, softcap, slopes, (const T*)gate, (size_t)gate_stride, out_scale)
   if (dtype == MS_F32) LAUNCH(float);
   else if (dtype == MS_BF16) LAUNCH(bf16);
   else return MS_BAD_ARG;

@@ -1,6 +1,6 @@
-// Layer norm with a weight and no bias on the float residual stream, the scaled sum that precedes it, and the gate of a
+// Layer norm with a weight and an optional bias on the float residual stream, the scaled sum that precedes it, and the gate of a
 // token's own side input into the stream.
-//   v = x[row] (+ scale o delta[row]);   out = w o (v - mean v) / sqrt(mean (v - mean v)^2 + eps)
+//   v = x[row] (+ scale o delta[row]);   out = w o (v - mean v) / sqrt(mean (v - mean v)^2 + eps) (+ b)
 // The row is held in LDS between the passes (mean, then the mean of the squared deviations, as the norm is defined; no
 // E[v^2] - E[v]^2), so out may be x itself.  Everything is float; out is rounded once.  Without a weight the kernel is
 // the scaled sum alone, and out (if given) takes the summed row rounded to its type: the operand of a product that reads
@@ -28,7 +28,8 @@ __device__ __forceinline__ void load_row(float* __restrict__ row, const float* _
 template <typename TD, typename TO>
 __global__ void __launch_bounds__(LN_THREADS)
 layer_norm_kernel(float* __restrict__ x, const TD* __restrict__ delta, const float* __restrict__ dscale,
-                  const float* __restrict__ w, const int* __restrict__ rows, TO* out, int H, float eps, int write_back) {
+                  const float* __restrict__ w, const float* __restrict__ b, const int* __restrict__ rows, TO* out, int H, float eps,
+                  int write_back) {
   extern __shared__ float row[];
   __shared__ float red[16];
   const size_t src = rows ? (size_t)rows[blockIdx.x] : (size_t)blockIdx.x;
@@ -45,7 +46,7 @@ layer_norm_kernel(float* __restrict__ x, const TD* __restrict__ delta, const flo
   const bool same = (const void*)o == (const void*)xr;     // the norm in place: x takes the normed row, not the sum
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     if (delta && write_back && !same) xr[i] = row[i];
-    if (w) o[i] = from_float<TO>((row[i] - mean) * inv * w[i]);
+    if (w) o[i] = from_float<TO>(b ? fmaf((row[i] - mean) * inv, w[i], b[i]) : (row[i] - mean) * inv * w[i]);
     else if (out) o[i] = from_float<TO>(row[i]);
   }
 }
@@ -68,16 +69,16 @@ side_gate_kernel(const T* __restrict__ z, size_t z_stride, const int* __restrict
 }  // namespace
 
 // x float [N, H]; delta (may be null) [N, H] of `delta_dtype`, dscale (may be null) float [H]; w (null: only the sum)
-// float [H]; rows (may be null) int32 [n_rows]: which rows of x; out [n_rows, H] of `out_dtype` (may be x for float).
+// float [H], b (may be null; only with w) float [H]; rows (may be null) int32 [n_rows]: which rows of x; out [n_rows, H] of `out_dtype` (may be x for float).
 extern "C" int ms_layer_norm(float* x, const void* delta, int delta_dtype, const float* dscale, const float* w,
-                             const int* rows, void* out, int n_rows, int H, float eps, int write_back, int out_dtype,
+                             const float* b, const int* rows, void* out, int n_rows, int H, float eps, int write_back, int out_dtype,
                              hipStream_t stream) {
   if (n_rows <= 0) return MS_OK;
-  if (H <= 0 || (w != nullptr && out == nullptr)) return MS_BAD_ARG;   // w null with out: the summed rows' rounded copy
+  if (H <= 0 || (w != nullptr && out == nullptr) || (b != nullptr && w == nullptr)) return MS_BAD_ARG;   // w null with out: the summed rows' rounded copy
   if (H > 16384) return MS_UNSUPPORTED;
   const size_t lds = (size_t)H * sizeof(float);
 #define LAUNCH(TD, TO)                                                                                               \
-  layer_norm_kernel<TD, TO><<<dim3(n_rows), dim3(LN_THREADS), lds, stream>>>(x, (const TD*)delta, dscale, w, rows,   \
+  layer_norm_kernel<TD, TO><<<dim3(n_rows), dim3(LN_THREADS), lds, stream>>>(x, (const TD*)delta, dscale, w, b, rows, \
                                                                              (TO*)out, H, eps, write_back)
   const bool dbf = delta != nullptr && delta_dtype == MS_BF16;
   if (delta != nullptr && delta_dtype != MS_BF16 && delta_dtype != MS_F32) return MS_BAD_ARG;

@@ -333,7 +333,8 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
 template <typename T>
 __global__ void gated_head_norm_kernel(const float* __restrict__ o, const float* __restrict__ w,
                                        const T* __restrict__ gate, size_t gate_stride, T* __restrict__ out,
-                                       long long items, int H, int E, float eps, int gate_silu) {
+                                       long long items, int H, int E, float eps, int gate_silu, int weight_per_head,
+                                       float scale) {
   const int lane = threadIdx.x & (MS_WAVE - 1);
   const long long item = (long long)blockIdx.x * (blockDim.x / MS_WAVE) + threadIdx.x / MS_WAVE;
   if (item >= items) return;
@@ -343,7 +344,8 @@ __global__ void gated_head_norm_kernel(const float* __restrict__ o, const float*
   float ss = 0.f;
   for (int i = lane; i < E; i += MS_WAVE) ss = fmaf(op[i], op[i], ss);
   ss = wave_sum(ss);
-  const float inv = 1.0f / sqrtf(ss / (float)E + eps);
+  const float inv = scale / sqrtf(ss / (float)E + eps);
+  if (weight_per_head) w += (size_t)h * E;
   const T* gp = gate + (size_t)n * gate_stride + (size_t)h * E;
   T* yp = out + (size_t)item * E;
   for (int i = lane; i < E; i += MS_WAVE) {
@@ -467,8 +469,8 @@ extern "C" int ms_gated_delta(const void* q, const void* k, const void* v, long 
 }
 
 extern "C" int ms_gated_head_norm(const float* o, const float* weight, const void* gate, long long gate_stride,
-                                  void* out, int n_tokens, int heads, int vdim, float eps, int gate_silu, int dtype,
-                                  hipStream_t stream) {
+                                  void* out, int n_tokens, int heads, int vdim, float eps, int gate_silu,
+                                  int weight_per_head, float scale, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return MS_OK;
   if (heads <= 0 || vdim <= 0) return MS_BAD_ARG;
   const long long items = (long long)n_tokens * heads;
@@ -476,10 +478,12 @@ extern "C" int ms_gated_head_norm(const float* o, const float* weight, const voi
   dim3 grid((unsigned)((items + waves - 1) / waves)), block(waves * MS_WAVE);
   if (dtype == MS_F32)
     gated_head_norm_kernel<float><<<grid, block, 0, stream>>>(o, weight, (const float*)gate, (size_t)gate_stride,
-                                                              (float*)out, items, heads, vdim, eps, gate_silu);
+                                                              (float*)out, items, heads, vdim, eps, gate_silu,
+                                                              weight_per_head, scale);
   else if (dtype == MS_BF16)
     gated_head_norm_kernel<bf16><<<grid, block, 0, stream>>>(o, weight, (const bf16*)gate, (size_t)gate_stride,
-                                                             (bf16*)out, items, heads, vdim, eps, gate_silu);
+                                                             (bf16*)out, items, heads, vdim, eps, gate_silu,
+                                                             weight_per_head, scale);
   else return MS_BAD_ARG;
   return ms_launch_status();
 }

@@ -62,7 +62,7 @@ _SIGNATURES = {
                         _c_int, _c_int, _c_ptr],
     "ms_paged_attention_generic": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                    _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ll, _c_float, _c_int, _c_int,
-                                   _c_ptr, _c_int, _c_ptr],
+                                   _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ll, _c_float, _c_int, _c_ptr],
     "ms_attention_mfma_supported": [_c_int, _c_int],
     "ms_paged_attention_mfma": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll,
                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr, _c_ptr],
@@ -77,7 +77,16 @@ _SIGNATURES = {
                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_gated_delta": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_int, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                        _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
-    "ms_gated_head_norm": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
+    "ms_gated_head_norm": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_float,
+                           _c_int, _c_ptr],
+    "ms_gelu_tanh_glu": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_decay_recurrence": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ll, _c_ll, _c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_float,
+                            _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_token_shift": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
+                       _c_int, _c_ptr],
+    "ms_pair_sum": [_c_ptr, _c_ptr, _c_float, _c_float, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_tanh": [_c_ptr, _c_ll, _c_int, _c_ptr],
+    "ms_concat_rows": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_xielu": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
     "ms_head_matmul": [_c_ptr, _c_ll, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_ll, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int,
                        _c_int, _c_int, _c_ptr],
@@ -96,12 +105,12 @@ _SIGNATURES = {
                         _c_ptr],
     "ms_add_rows": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "ms_qk_norm_store": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_float, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
-                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_ptr],
     "ms_selective_scan": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_ptr,
                           _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_gelu": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
     "ms_moe_route": [_c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
-    "ms_layer_norm": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
+    "ms_layer_norm": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "ms_side_gate": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "ms_mingru_chunk": [],
     "ms_mingru_scan": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_ptr,
@@ -742,7 +751,9 @@ def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
                             token_req: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, num_heads: int,
                             scale: float, window: Optional[int] = None, v_transposed: bool = False,
                             table_rows: Optional[torch.Tensor] = None,
-                            n_live_tokens: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+                            n_live_tokens: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None,
+                            softcap: float = 0.0, slopes: Optional[torch.Tensor] = None,
+                            gate: Optional[torch.Tensor] = None, out_scale: float = 1.0) -> torch.Tensor:
     """out[n, h] = softmax(scale * q[n, h] . K[keys visible to n]) V, keys read in place from pages.
 
     q: [N, >= nh * d] (a row slice of the fused projection is fine), out [N, nh * d],
@@ -752,7 +763,9 @@ def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
     pages are row ``table_rows[token_req[n]]`` of the table (row token_req[n] without ``table_rows``).  With
     ``n_live_tokens`` (a device int) tokens from that index on are left alone.  Values may have another size than
     keys (the value pages say which; out is then [N, nh * that size]).  ``sink`` float [nh]: exp(sink[h]) joins the
-    denominator of head h's softmax."""
+    denominator of head h's softmax.  ``softcap`` > 0: a scaled score s becomes softcap * tanh(s / softcap).  ``slopes``
+    float [nh]: slopes[h] * (positions[n] - key's position) is taken off the score (after the cap).  ``gate`` [N, nh] (rows
+    may be slices): head h's result is multiplied by sigmoid(gate[n, h]); ``out_scale`` multiplies every result."""
     _check(k_pages, "k_pages")
     P, nkv, page_size, d = k_pages.shape
     _check(v_pages, "v_pages", k_pages.dtype, (P, nkv, None, None))
@@ -776,11 +789,17 @@ def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
         _check(n_live_tokens, "n_live_tokens", torch.int32, (1,))
     if num_heads % nkv:
         raise ValueError(f"{num_heads} query heads cannot share {nkv} key/value heads")
+    if slopes is not None:
+        _check(slopes, "slopes", torch.float32, (num_heads,))
+    gate_stride = _rows2d(gate, "gate", q.dtype, num_heads) if gate is not None else 0
+    if gate is not None and gate.shape[0] != N:
+        raise ValueError("gate must have a row per token")
     _call("ms_paged_attention_generic", q.data_ptr(), q.stride(0) if N > 1 else q.shape[1], k_pages.data_ptr(),
           v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], _ptr(table_rows), _ptr(n_live_tokens),
           token_req.data_ptr(), positions.data_ptr(),
           out.data_ptr(), num_heads * dv, N, num_heads, nkv, d, dv, page_size, P, float(scale), int(window or 0),
-          int(v_transposed), _ptr(sink), _code(q.dtype), _stream())
+          int(v_transposed), _ptr(sink), float(softcap or 0.0), _ptr(slopes), _ptr(gate), gate_stride, float(out_scale),
+          _code(q.dtype), _stream())
     return out
 
 
@@ -893,16 +912,20 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.
 
 
 def paged_attention(q: torch.Tensor, kv, ctx, out: torch.Tensor, num_heads: int, scale: float,
-                    window: Optional[int] = None, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    window: Optional[int] = None, sink: Optional[torch.Tensor] = None, softcap: float = 0.0,
+                    slopes: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                    out_scale: float = 1.0) -> torch.Tensor:
     """Attention of a step's tokens (``ctx``: its StepContext) over a run's pages (``kv``: its KVView).
     bfloat16 with transposed value pages and a head size the matrix-core kernel has goes there; everything
     else (float32, other head sizes, values of another size than keys, small pages) goes to the generic kernel.
     ``sink`` float [num_heads]: exp(sink[h]) joins the denominator of head h's softmax."""
     d, page_size = kv.k_pages.shape[3], kv.k_pages.shape[2]
     dv = kv.v_pages.shape[2] if kv.v_transposed else kv.v_pages.shape[3]
-    if dv != d:
+    if dv != d or softcap or slopes is not None or gate is not None or out_scale != 1.0:
+        # capped scores, a distance penalty and an output gate are the generic kernel's
         return paged_attention_generic(q, kv.k_pages, kv.v_pages, kv.block_table, ctx.token_req, ctx.positions, out,
-                                       num_heads, scale, window, kv.v_transposed, kv.table_rows, ctx.n_live_tokens, sink)
+                                       num_heads, scale, window, kv.v_transposed, kv.table_rows, ctx.n_live_tokens, sink,
+                                       softcap, slopes, gate, out_scale)
     if q.dtype == torch.bfloat16 and not (kv.v_transposed and attention_mfma_supported(d, page_size)):
         _say_once(("attention", d, page_size),
                   f"bfloat16 attention with head size {d} and pages of {page_size} tokens runs on the vector-ALU kernel: "
@@ -993,18 +1016,109 @@ def gated_delta(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tens
 
 
 def gated_head_norm(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, out: torch.Tensor, heads: int, vdim: int,
-                    eps: float, gate_act: str = "sigmoid") -> torch.Tensor:
-    """out[n, h] = o[n, h] / sqrt(mean(o[n, h]^2) + eps) * weight * act(gate[n, h]), act "sigmoid" or "silu";
-    o float [N, heads * vdim]."""
+                    eps: float, gate_act: str = "sigmoid", scale: float = 1.0) -> torch.Tensor:
+    """out[n, h] = scale * o[n, h] / sqrt(mean(o[n, h]^2) + eps) * weight * act(gate[n, h]), act "sigmoid" or "silu";
+    o float [N, heads * vdim]; weight float [vdim], shared by the heads, or [heads * vdim], every head its own."""
     if gate_act not in ("sigmoid", "silu"):
         raise ValueError(f"the read-out's gate is 'sigmoid' or 'silu', not {gate_act!r}")
     N = o.shape[0]
     _check(o, "o", torch.float32, (N, heads * vdim))
-    _check(weight, "weight", torch.float32, (vdim,))
+    per_head = weight.numel() == heads * vdim and heads > 1
+    _check(weight, "weight", torch.float32, (heads * vdim if per_head else vdim,))
     gs = _rows2d(gate, "gate", out.dtype, heads * vdim)
     _check(out, "out", None, (N, heads * vdim))
     _call("ms_gated_head_norm", o.data_ptr(), weight.data_ptr(), gate.data_ptr(), gs, out.data_ptr(), N, heads, vdim,
-          float(eps), int(gate_act == "silu"), _code(out.dtype), _stream())
+          float(eps), int(gate_act == "silu"), int(per_head), float(scale), _code(out.dtype), _stream())
+    return out
+
+
+DECAY_SIGMOID_ROOT, DECAY_DOUBLE_EXP = 0, 1
+
+
+def decay_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor, z_bias: Optional[torch.Tensor],
+                     state: torch.Tensor, ctx, out: torch.Tensor, heads: int, dim: int, vdim: int, decay: int,
+                     tau: float = 1.0, bonus: Optional[torch.Tensor] = None, q_scale: float = 1.0) -> torch.Tensor:
+    """A recurrence with a decay per head and key channel over the step's portions, from and into ``state`` float
+    [slots, heads, dim, vdim]: per head and token  S <- diag(w) S + k v^T  and  o = S^T (q_scale q)  read after the write;
+    with ``bonus`` u float [heads * dim] the read comes first and weights the current token:
+    o = (S + diag(u) k v^T)^T (q_scale q), then the write.  The decay is made from z float [N, heads * dim] (+ ``z_bias``
+    float [heads * dim]): DECAY_SIGMOID_ROOT: w = sigmoid(z)^(1 / tau); DECAY_DOUBLE_EXP: w = exp(-exp(z)).  q, k
+    [N, heads * dim] and v [N, heads * vdim] may be row slices; out float [N, heads * vdim]."""
+    N = q.shape[0]
+    sq = _rows2d(q, "q", None, heads * dim)
+    sk = _rows2d(k, "k", q.dtype, heads * dim)
+    sv = _rows2d(v, "v", q.dtype, heads * vdim)
+    if k.shape[0] != N or v.shape[0] != N:
+        raise ValueError("q, k and v must have a row per token")
+    _check(z, "z", torch.float32, (N, heads * dim))
+    if z_bias is not None:
+        _check(z_bias, "z_bias", torch.float32, (heads * dim,))
+    if bonus is not None:
+        _check(bonus, "bonus", torch.float32, (heads * dim,))
+    if decay not in (DECAY_SIGMOID_ROOT, DECAY_DOUBLE_EXP):
+        raise ValueError("decay is DECAY_SIGMOID_ROOT or DECAY_DOUBLE_EXP")
+    if decay == DECAY_SIGMOID_ROOT and not tau > 0:
+        raise ValueError("tau must be positive")
+    _check(state, "state", torch.float32, (None, heads, dim, vdim))
+    _check(out, "out", torch.float32, (N, heads * vdim))
+    R = ctx.num_requests
+    _check(ctx.q_start, "q_start", torch.int32, (R + 1,))
+    _check(ctx.state_slots, "state_slots", torch.int32, (R,))
+    _call("ms_decay_recurrence", q.data_ptr(), k.data_ptr(), v.data_ptr(), sq, sk, sv, z.data_ptr(), _ptr(z_bias), int(decay),
+          1.0 / float(tau), _ptr(bonus), float(q_scale), state.data_ptr(), ctx.q_start.data_ptr(), ctx.state_slots.data_ptr(),
+          out.data_ptr(), R, heads, dim, vdim, _code(q.dtype), _stream())
+    return out
+
+
+def token_shift(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, ctx, out: torch.Tensor) -> torch.Tensor:
+    """out[m, n] = h[n] + (h'[n] - h[n]) o mu[m] for the step ``ctx`` describes, h' the previous token's row of h: the row
+    before within a portion, ``state`` [slots, 1, W] (the request's slot; zero at a request's start) for a portion's first
+    token.  The state then becomes the last row of every request's portion.  mu float [M, W]; out [M, N, W] of h's type."""
+    N, W = h.shape
+    hs = _rows2d(h, "h")
+    _check(mu, "mu", torch.float32, (None, W))
+    M = mu.shape[0]
+    _check(state, "state", h.dtype, (None, 1, W))
+    _check(out, "out", h.dtype, (M, N, W))
+    R = ctx.num_requests
+    _check(ctx.token_req, "token_req", torch.int32, (N,))
+    _check(ctx.q_start, "q_start", torch.int32, (R + 1,))
+    _check(ctx.state_slots, "state_slots", torch.int32, (R,))
+    _call("ms_token_shift", h.data_ptr(), hs, mu.data_ptr(), state.data_ptr(), ctx.token_req.data_ptr(), ctx.q_start.data_ptr(),
+          ctx.state_slots.data_ptr(), _ptr(ctx.n_live_tokens), out.data_ptr(), N, R, W, M, _code(h.dtype), _stream())
+    return out
+
+
+def pair_sum(x: torch.Tensor, a: torch.Tensor, b: torch.Tensor, scale_a: float = 1.0, scale_b: float = 1.0,
+             norm_a: Optional[torch.Tensor] = None, norm_b: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
+    """x[n] += scale_a f(a[n]) + scale_b g(b[n]), in place on the float residual stream; f is the identity, or with
+    ``norm_a`` (float [W]) the row divided by its root mean square (eps inside the root) times that weight; g likewise."""
+    _check(x, "x", torch.float32)
+    N, W = x.shape
+    _check(a, "a", None, (N, W))
+    _check(b, "b", a.dtype, (N, W))
+    for w, name in ((norm_a, "norm_a"), (norm_b, "norm_b")):
+        if w is not None:
+            _check(w, name, torch.float32, (W,))
+    _call("ms_pair_sum", a.data_ptr(), b.data_ptr(), float(scale_a), float(scale_b), _ptr(norm_a), _ptr(norm_b), float(eps),
+          x.data_ptr(), N, W, _code(a.dtype), _stream())
+    return x
+
+
+def tanh_(x: torch.Tensor) -> torch.Tensor:
+    """x <- tanh(x), in place (computed in float, rounded once)."""
+    _check(x, "x")
+    _call("ms_tanh", x.data_ptr(), x.numel(), _code(x.dtype), _stream())
+    return x
+
+
+def concat_rows(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[n] = [a[n] | b[n]] in out's type; a [N, Wa] and b [N, Wb] float."""
+    _check(a, "a", torch.float32)
+    _check(b, "b", torch.float32, (a.shape[0], None))
+    _check(out, "out", None, (a.shape[0], a.shape[1] + b.shape[1]))
+    _call("ms_concat_rows", a.data_ptr(), b.data_ptr(), out.data_ptr(), a.shape[0], a.shape[1], b.shape[1], _code(out.dtype),
+          _stream())
     return out
 
 
@@ -1192,9 +1306,12 @@ def qk_norm_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
                   q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
                   positions: Optional[torch.Tensor] = None, coef: float = 0.0, every: int = 1,
                   slot_mapping: Optional[torch.Tensor] = None, k_pages: Optional[torch.Tensor] = None,
-                  v_pages: Optional[torch.Tensor] = None, v_transposed: bool = False) -> torch.Tensor:
+                  v_pages: Optional[torch.Tensor] = None, v_transposed: bool = False, unit_norm: bool = False,
+                  inv_freq: Optional[torch.Tensor] = None, rot_dim: int = 0) -> torch.Tensor:
     """In place on ``qkv`` [N, nh d + nkv d + nkv dv]: the RMS norm of every q and k head with the weights [d] (None: no
-    norm), q of the token at position p times 1 + coef * ln(floor((p + 1) / every) + 1); then k and v go into the pages
+    norm, or with ``unit_norm`` the division by the root mean square alone), q of the token at position p times
+    1 + coef * ln(floor((p + 1) / every) + 1); with ``rot_dim`` > 0 entry i and entry i + rot_dim / 2 of every q and k head
+    then turn by position * inv_freq[i] (float [rot_dim / 2]); then k and v go into the pages
     ([P, nkv, page, d] and [P, nkv, page, dv], or values [P, nkv, dv, page] with ``v_transposed``) at ``slot_mapping``."""
     width = (num_heads + num_kv_heads) * head_dim + num_kv_heads * value_dim
     stride = _rows2d(qkv, "qkv", None, width)
@@ -1206,6 +1323,11 @@ def qk_norm_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
         _check(positions, "positions", torch.int32, (N,))
         if every <= 0:
             raise ValueError("the query temperature's period must be positive")
+    if rot_dim:
+        if rot_dim % 2 or not 0 < rot_dim <= head_dim:
+            raise ValueError(f"{rot_dim} rotated entries must be even and within the head's {head_dim}")
+        _check(positions, "positions", torch.int32, (N,))
+        _check(inv_freq, "inv_freq", torch.float32, (rot_dim // 2,))
     page_size = 0
     if k_pages is not None:
         _check(k_pages, "k_pages", qkv.dtype, (None, num_kv_heads, None, head_dim))
@@ -1214,7 +1336,8 @@ def qk_norm_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
         _check(slot_mapping, "slot_mapping", torch.int32, (N,))
     _call("ms_qk_norm_store", qkv.data_ptr(), stride, _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(positions), float(coef),
           int(every), _ptr(slot_mapping), _ptr(k_pages), _ptr(v_pages), N, num_heads, num_kv_heads, head_dim, value_dim,
-          page_size, int(bool(v_transposed)), _code(qkv.dtype), _stream())
+          page_size, int(bool(v_transposed)), int(bool(unit_norm)), _ptr(inv_freq) if rot_dim else None, int(rot_dim),
+          _code(qkv.dtype), _stream())
     return qkv
 
 
@@ -1392,8 +1515,8 @@ def moe_combine(part: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, h:
 # ------------------------------------------------------------------------------------------------ layer norm, side input
 def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out: Optional[torch.Tensor],
                delta: Optional[torch.Tensor] = None, delta_scale: Optional[torch.Tensor] = None,
-               rows: Optional[torch.Tensor] = None, write_back: bool = True):
-    """out[r] = weight * (v - mean v) / sqrt(mean (v - mean v)^2 + eps) with v = x[rows[r]] (+ delta_scale o delta[rows[r]]).
+               rows: Optional[torch.Tensor] = None, write_back: bool = True, bias: Optional[torch.Tensor] = None):
+    """out[r] = weight * (v - mean v) / sqrt(mean (v - mean v)^2 + eps) (+ bias) with v = x[rows[r]] (+ delta_scale o delta[rows[r]]).
     x float32 [N, H] is the residual stream; with ``delta`` [N, H] the sum is written back to x (unless ``write_back`` is
     False).  ``weight`` None: only the sum, and ``out`` (if given) takes the summed rows rounded to its type.  ``out`` may
     be x itself (float): the rows are normed in place."""
@@ -1405,6 +1528,10 @@ def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out:
         n_rows = rows.numel()
     if weight is not None:
         _check(weight, "weight", torch.float32, (H,))
+    if bias is not None:
+        if weight is None:
+            raise ValueError("a bias without a weight")
+        _check(bias, "bias", torch.float32, (H,))
     if weight is not None or out is not None:
         _check(out, "out", None, (n_rows, H))
     dcode = 0
@@ -1415,7 +1542,7 @@ def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out:
             _check(delta_scale, "delta_scale", torch.float32, (H,))
     elif delta_scale is not None:
         raise ValueError("a scale without an addend")
-    _call("ms_layer_norm", x.data_ptr(), _ptr(delta), dcode, _ptr(delta_scale), _ptr(weight), _ptr(rows),
+    _call("ms_layer_norm", x.data_ptr(), _ptr(delta), dcode, _ptr(delta_scale), _ptr(weight), _ptr(bias), _ptr(rows),
           _ptr(out), n_rows, H, float(eps), int(write_back), _code(out.dtype) if out is not None else F32, _stream())
     return out
 
@@ -1597,6 +1724,19 @@ def clamped_glu(gu: torch.Tensor, out: torch.Tensor, limit: float, alpha: float 
         raise ValueError("out has one row per row of gu")
     _call("ms_clamped_glu", gu.data_ptr(), s_in, out.data_ptr(), s_out, gu.shape[0], F, float(limit), float(alpha),
           _code(gu.dtype), _stream())
+    return out
+
+
+def gelu_tanh_glu(gu: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[n, f] = gelu_tanh(g) * u for gu [N, 2F] with gate and up interleaved (g0, u0, g1, u1, ...), the tanh form of the
+    gelu: z/2 (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))."""
+    N = gu.shape[0]
+    F = gu.shape[1] // 2
+    gs = _rows2d(gu, "gu", None, 2 * F)
+    os_ = _rows2d(out, "out", gu.dtype, F)
+    if out.shape[0] != N:
+        raise ValueError("out must have a row per row of gu")
+    _call("ms_gelu_tanh_glu", gu.data_ptr(), gs, out.data_ptr(), os_, N, F, _code(gu.dtype), _stream())
     return out
 
 

@@ -5,8 +5,13 @@ attention read in place from the pages, output projection.  Query head h uses ke
 h // (num_heads // num_kv_heads) (src/miniserve/model.py:137-139).  Scores, softmax and the weighted
 sum are float.  ``window`` limits a query to the last ``window`` keys (None: all).  ``value_dim``: values of another
 size than queries and keys.  ``sink``: a learned number per query head (tensor ``sink`` [heads]) whose exponential joins
-the softmax's denominator; it has no key and no value and is not scaled.  ``names``: the tensors' names after the prefix,
-{"q", "k", "v", "o", "sink"} -> name; biases are the weight's name with ".bias" for ".weight".
+the softmax's denominator; it has no key and no value and is not scaled; ``sink="zero"``: the same with the constant 0 for
+every head and no tensor (one is added to the denominator).  ``softcap`` c: a scaled score s becomes c tanh(s / c).
+``slope_base`` b: head h of H takes slope_h (i - j) off the score of key j for query i, slope_h = 2^(-b (h + 1) / H) (after the
+cap).  ``gate``: a projection [heads, hidden] (tensor "gate") whose sigmoid multiplies every head's result, one number per
+token and head, before the output projection; it rides on the packed q/k/v product.  ``out_scale`` multiplies the heads'
+results.  ``names``: the tensors' names after the prefix, {"q", "k", "v", "o", "sink", "gate"} -> name; biases are the weight's
+name with ".bias" for ".weight", or the weight's name followed by ``bias_suffix``.
 """
 from __future__ import annotations
 
@@ -18,7 +23,8 @@ from ..kernels import linear, ops
 from ..weights.spec import TensorSpec
 from .base import CacheNeed, KVNeed, Mixer, PageTensor, register_part
 
-_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight", "sink": "sink"}
+_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight", "sink": "sink",
+          "gate": "gate"}
 
 
 class GQAttention(Mixer):
@@ -26,7 +32,9 @@ class GQAttention(Mixer):
 
     def __init__(self, prefix: str, position, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  scale: float, qkv_bias: bool = True, out_bias: bool = False, window: Optional[int] = None,
-                 value_dim: Optional[int] = None, sink: bool = False, names=None):
+                 value_dim: Optional[int] = None, sink=False, names=None, softcap: Optional[float] = None,
+                 slope_base: Optional[float] = None, gate: bool = False, out_scale: float = 1.0,
+                 bias_suffix: Optional[str] = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads cannot share {num_kv_heads} key/value heads")
         if not 0 < head_dim <= 256:
@@ -42,11 +50,27 @@ class GQAttention(Mixer):
         if self.value_dim != head_dim and not getattr(position, "takes_value_dim", False):
             raise ValueError("values of another size than keys need a position encoding that stores them "
                              "(one with takes_value_dim)")
-        self.sink = bool(sink)
+        if sink not in (False, True, "zero"):
+            raise ValueError(f"sink is False, True (a learned number per head) or 'zero', got {sink!r}")
+        self.sink = sink is True
+        self.zero_sink = sink == "zero"
+        if softcap is not None and not softcap > 0:
+            raise ValueError("softcap must be positive")
+        self.softcap = float(softcap) if softcap is not None else 0.0
+        self.slope_base = float(slope_base) if slope_base is not None else None
+        self.gate, self.out_scale, self.bias_suffix = bool(gate), float(out_scale), bias_suffix
         self.names = dict(_NAMES, **dict(names or {}))
+        self.slopes = self.w_gate_rows = None
+
+    @property
+    def _extras(self) -> bool:
+        """Whether attention needs more than the causal (windowed) softmax with an optional sink."""
+        return bool(self.softcap or self.slope_base is not None or self.gate or self.out_scale != 1.0)
 
     def _bias_name(self, which: str) -> str:
         name = self.names[which]
+        if self.bias_suffix is not None:
+            return name + self.bias_suffix
         return name[:-len(".weight")] + ".bias" if name.endswith(".weight") else name + ".bias"
 
     # ---- weights
@@ -62,6 +86,8 @@ class GQAttention(Mixer):
             specs.append(TensorSpec(p + self._bias_name("o"), (H,), "bias"))
         if self.sink:
             specs.append(TensorSpec(p + self.names["sink"], (self.num_heads,), "bias"))
+        if self.gate:
+            specs.append(TensorSpec(p + self.names["gate"], (self.num_heads, H)))
         if self.position is not None:
             specs += self.position.tensor_specs()
         return specs
@@ -71,12 +97,24 @@ class GQAttention(Mixer):
         by_name = {s.name: s for s in GQAttention.tensor_specs(self)}
         p = self.prefix
         w = [get(by_name[p + self.names[n]]) for n in ("q", "k", "v")]
+        if self.gate:       # the gate's rows ride on the packed product, after q, k and v
+            w.append(get(by_name[p + self.names["gate"]]))
         self.w_qkv = linear.prepare_weight(torch.cat(w, dim=0))
-        self.b_qkv = torch.cat([get(by_name[p + self._bias_name(n)]) for n in ("q", "k", "v")]).contiguous() \
-            if self.qkv_bias else None
+        self.b_qkv = None
+        if self.qkv_bias:
+            b = [get(by_name[p + self._bias_name(n)]) for n in ("q", "k", "v")]
+            if self.gate:
+                b.append(torch.zeros(self.num_heads, dtype=b[0].dtype, device=b[0].device))
+            self.b_qkv = torch.cat(b).contiguous()
         self.w_o = linear.prepare_weight(get(by_name[p + self.names["o"]]))
         self.b_o = get(by_name[p + self._bias_name("o")]) if self.out_bias else None
         self.sink_w = get(by_name[p + self.names["sink"]]) if self.sink else None
+        if self.zero_sink:
+            self.sink_w = torch.zeros(self.num_heads, dtype=torch.float32, device=rt.device)
+        if self.slope_base is not None:
+            H = self.num_heads
+            self.slopes = torch.tensor([2.0 ** (-self.slope_base * (h + 1) / H) for h in range(H)], dtype=torch.float64) \
+                .to(torch.float32).to(rt.device)
         if self.position is not None:
             self.position.load(get, rt)
 
@@ -84,7 +122,7 @@ class GQAttention(Mixer):
     def cache_need(self):
         # in bfloat16 the matrix-core attention reads value pages as an operand as they lie, transposed, which it
         # can for pages of a multiple of 16 tokens
-        if self.value_dim == self.head_dim:
+        if self.value_dim == self.head_dim and not self._extras:
             return KVNeed(self.num_kv_heads, self.head_dim, self.window, transpose_values_at=16,
                           transpose_values_in=torch.bfloat16)
         return CacheNeed((PageTensor("k", self.num_kv_heads, self.head_dim),
@@ -98,6 +136,8 @@ class GQAttention(Mixer):
         if kv is None:
             raise RuntimeError("attention needs a key/value cache view")
         nh, nkv, d, dv = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
+        if self.gate:
+            return self._forward_gated(h, ctx, kv, x)
         q = None
         if self.position is not None and dv == d:
             q = self.position.project_encode_store(h, self.w_qkv, self.b_qkv, nh, nkv, d, ctx, kv)
@@ -116,7 +156,28 @@ class GQAttention(Mixer):
             elif kv.store:
                 ops.rope_store(q, nh, nkv, d, 0, None, None, kv.slot_mapping, kv.k_pages, kv.v_pages, kv.v_transposed)
         out = self.rt.empty(ctx.num_tokens, nh * dv)
-        ops.paged_attention(q, kv, ctx, out, nh, self.scale, self.window, self.sink_w)
+        ops.paged_attention(q, kv, ctx, out, nh, self.scale, self.window, self.sink_w, self.softcap, self.slopes, None,
+                            self.out_scale)
+        return linear.linear_residual(out, self.w_o, self.b_o, x)
+
+    def _forward_gated(self, h, ctx, kv, x):
+        """With an output gate: one product for q, k, v and the gate's numbers; the position encoding works on the first
+        columns, the attention kernel reads the last ones."""
+        nh, nkv, d, dv = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
+        width = (nh + nkv) * d + nkv * dv
+        proj = linear.linear(h, self.w_qkv, bias=self.b_qkv)
+        qkv = proj[:, :width]
+        if self.position is None:
+            if kv.store:
+                ops.qk_norm_store(qkv, nh, nkv, d, dv, None, None, 0.0, slot_mapping=kv.slot_mapping, k_pages=kv.k_pages,
+                                  v_pages=kv.v_pages, v_transposed=kv.v_transposed)
+        elif dv != d or getattr(self.position, "takes_value_dim", False):
+            self.position.encode_and_store(qkv, nh, nkv, d, ctx, kv, value_dim=dv)
+        else:
+            self.position.encode_and_store(qkv, nh, nkv, d, ctx, kv)
+        out = self.rt.empty(ctx.num_tokens, nh * dv)
+        ops.paged_attention(qkv, kv, ctx, out, nh, self.scale, self.window, self.sink_w, self.softcap, self.slopes,
+                            proj[:, width:], self.out_scale)
         return linear.linear_residual(out, self.w_o, self.b_o, x)
 
 

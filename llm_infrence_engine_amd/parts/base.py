@@ -442,8 +442,9 @@ class PassEntry(Part):
 
     keeps_embedding = False    # True: ``forward`` wants the residual stream as the embedding left it
 
-    def forward(self, x: torch.Tensor, kept: Optional[torch.Tensor], t: int) -> None:
-        """Change x [N, H] (float) in place before pass ``t`` (0, 1, ...); ``kept``: the embedding's output, if asked for."""
+    def forward(self, x: torch.Tensor, kept: Optional[torch.Tensor], t: int) -> Optional[torch.Tensor]:
+        """Change x [N, H] (float) in place before pass ``t`` (0, 1, ...) and return None, or return the new residual
+        stream (float [N, H], another tensor); ``kept``: the embedding's output, if asked for."""
         raise NotImplementedError
 
 

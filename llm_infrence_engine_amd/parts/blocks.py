@@ -25,7 +25,8 @@ class PreNormResidual(Block):
 class ParallelResidual(Block):
     """x <- x + mixer(f(norm1(x))) + feed_forward(norm2(x)): both branches read the same x.  ``input_filter``
     (optional) is a map over time laid before the mixer's input, f; without a feed-forward the layer is
-    x <- x + mixer(f(norm1(x)))."""
+    x <- x + mixer(f(norm1(x))).  A layer with a feed-forward and no ``feed_forward_norm`` has one norm that both
+    branches read: x <- x + mixer(f(h)) + feed_forward(h), h = norm1(x)."""
 
     takes = {"position": "position", "mixer_norm": "norm", "input_filter": "filter", "mixer": "mixer",
              "feed_forward_norm": "norm", "feed_forward": "feed_forward"}
@@ -33,7 +34,9 @@ class ParallelResidual(Block):
 
     def forward(self, x, pending, ctx, kv, state):
         # x holds the sum both branches read before either adds to it; the two norms share their pass over x
-        if self.feed_forward is not None and hasattr(self.mixer_norm, "forward_pair"):
+        if self.feed_forward is not None and self.feed_forward_norm is None:
+            h = h2 = self.mixer_norm.forward(x, delta=pending)
+        elif self.feed_forward is not None and hasattr(self.mixer_norm, "forward_pair"):
             h, h2 = self.mixer_norm.forward_pair(self.feed_forward_norm, x, delta=pending)
         else:
             h = self.mixer_norm.forward(x, delta=pending)

@@ -81,6 +81,29 @@ class PassStep(PassEntry):
         ops.add_rows(x, kept if (t > 0 and self.keeps_embedding) else None, self.step[t])
 
 
+class PassMix(PassEntry):
+    """Before every pass (the first too): x <- M [x ; e], with e the residual stream as the embedding left it and M a
+    stored matrix [hidden_size, 2 hidden_size] (tensor ``name``) whose first half of columns meets x.  The product reads
+    x and e rounded to the matrices' type and leaves as float, the new residual stream."""
+
+    keeps_embedding = True
+
+    def __init__(self, prefix: str, hidden_size: int, name: str = "in"):
+        self.prefix, self.hidden_size, self.name = prefix, hidden_size, name
+
+    def tensor_specs(self):
+        return [TensorSpec(self.prefix + self.name, (self.hidden_size, 2 * self.hidden_size))]
+
+    def load(self, get, rt):
+        self.rt = rt
+        self.weight = linear.prepare_weight(get(self.tensor_specs()[0]))
+
+    def forward(self, x, kept, t):
+        both = ops.concat_rows(x, kept, self.rt.empty(x.shape[0], 2 * self.hidden_size))
+        return linear.linear(both, self.weight, out_dtype=torch.float32)
+
+
 register_part("pass_entry", "pass_step", PassStep)
+register_part("pass_entry", "pass_mix", PassMix)
 register_part("embedding", "token_embedding", TokenEmbedding)
 register_part("head", "lm_head", LMHead)

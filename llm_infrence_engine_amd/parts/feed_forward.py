@@ -91,6 +91,43 @@ class ClampedGLU(FeedForward):
         return linear.linear(act, self.w_down)
 
 
+class GatedGLU(FeedForward):
+    """down(act(gate(x)) * up(x)), no biases, with ``activation`` "gelu_tanh": z/2 (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))),
+    or "silu" (the gated feed-forward above, under other tensor names).  Gate and up are one packed product (rows
+    interleaved); the activation is float."""
+
+    ACTIVATIONS = ("gelu_tanh", "silu")
+
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, activation: str = "gelu_tanh",
+                 gate_name: str = "gate", up_name: str = "up", down_name: str = "down"):
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"no activation {activation!r}; there are {', '.join(self.ACTIVATIONS)}")
+        self.prefix, self.hidden_size, self.intermediate_size, self.activation = prefix, hidden_size, intermediate_size, activation
+        self.gate_name, self.up_name, self.down_name = gate_name, up_name, down_name
+
+    def tensor_specs(self):
+        p, H, I = self.prefix, self.hidden_size, self.intermediate_size
+        return [TensorSpec(p + self.gate_name, (I, H)), TensorSpec(p + self.up_name, (I, H)), TensorSpec(p + self.down_name, (H, I))]
+
+    def load(self, get, rt):
+        self.rt = rt
+        g, u, d = (get(s) for s in self.tensor_specs())
+        self.w_gate_up = linear.interleave_rows(g, u)
+        self.w_down = linear.prepare_weight(d)
+
+    def forward(self, h, ctx):
+        return self.forward_residual(h, ctx, None)
+
+    def forward_residual(self, h, ctx, x):
+        if self.activation == "silu":
+            act = linear.linear_swiglu(h, self.w_gate_up)
+        else:
+            gu = linear.linear(h, self.w_gate_up)
+            act = ops.gelu_tanh_glu(gu, self.rt.empty(gu.shape[0], self.intermediate_size))
+        return linear.linear_residual(act, self.w_down, None, x)
+
+
 register_part("feed_forward", "swiglu", SwiGLU)
+register_part("feed_forward", "gated_glu", GatedGLU)
 register_part("feed_forward", "clamped_glu", ClampedGLU)
 register_part("feed_forward", "dense_act", DenseAct)

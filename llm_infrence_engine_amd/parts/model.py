@@ -13,8 +13,8 @@ import torch
 from ..config.spec import ModelSpec
 from ..weights.reader import CheckpointReader, place
 from ..weights.spec import TensorSpec
-from . import (attention, blocks, delta, ends, experts, feed_forward, filters, latent, mingru, norms,  # noqa: F401
-               pooled_attention, positions, scan, side)      # (register the built-in parts)
+from . import (attention, blocks, delta, ends, experts, feed_forward, filters, latent, linear_attention, mingru,  # noqa: F401
+               norms, pooled_attention, positions, scan, side, side_by_side)      # (register the built-in parts)
 from .base import KVView, Runtime, StateView, StepContext, build_part, part_class, weakest
 
 
@@ -103,7 +103,8 @@ class Model:
 
                     ops.residual_add(x, pending)
                     pending = None
-                self.pass_entry.forward(x, kept, run.opens_pass)
+                new = self.pass_entry.forward(x, kept, run.opens_pass)
+                x = x if new is None else new
             c = caches[i]
             pending = self.layers[run.layer].forward(x, pending, ctx, c.kv, c.state)
         return x, pending

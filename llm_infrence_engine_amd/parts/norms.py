@@ -71,31 +71,43 @@ class RMSNorm(Norm):
 
 
 class LayerNorm(Norm):
-    """y = weight * (x - mean x) / sqrt(mean (x - mean x)^2 + eps): a weight and no bias, computed in float on the float
-    residual stream.  ``forward`` also takes ``delta_scale``, a float vector the addend is multiplied by, element by
+    """y = weight * (x - mean x) / sqrt(mean (x - mean x)^2 + eps) (+ bias), computed in float on the float residual
+    stream.  ``bias_name``: the bias tensor's name (None: the norm has none).  ``gain``: a constant the result is
+    multiplied by, folded into weight and bias once, in float, when they are loaded (the scale of the logits, for a
+    model's last norm).  ``forward`` also takes ``delta_scale``, a float vector the addend is multiplied by, element by
     element, on its way into x (a layer's scale)."""
 
     takes_delta_scale = True
 
-    def __init__(self, prefix: str, size: int, eps: float, name: str = "weight"):
+    def __init__(self, prefix: str, size: int, eps: float, name: str = "weight", bias_name: str = None, gain: float = 1.0):
         self.prefix, self.size, self.eps, self.name = prefix, size, float(eps), name
+        self.bias_name, self.gain = bias_name, float(gain)
+        self.bias = None
 
     def tensor_specs(self):
-        return [TensorSpec(self.prefix + self.name, (self.size,), "norm")]
+        specs = [TensorSpec(self.prefix + self.name, (self.size,), "norm")]
+        if self.bias_name is not None:
+            specs.append(TensorSpec(self.prefix + self.bias_name, (self.size,), "bias"))
+        return specs
 
     def load(self, get, rt):
         self.rt = rt
-        self.weight = get(self.tensor_specs()[0])
+        specs = self.tensor_specs()
+        self.weight = get(specs[0])
+        self.bias = get(specs[1]) if self.bias_name is not None else None
+        if self.gain != 1.0:
+            self.weight = (self.weight * self.gain).contiguous()
+            self.bias = (self.bias * self.gain).contiguous() if self.bias is not None else None
 
     def forward(self, x, delta=None, rows=None, write_back=True, delta_scale=None):
         n = x.shape[0] if rows is None else rows.numel()
         out = self.rt.empty(n, self.size)
         return ops.layer_norm(x, self.weight, self.eps, out, delta=delta, delta_scale=delta_scale, rows=rows,
-                              write_back=write_back)
+                              write_back=write_back, bias=self.bias)
 
     def normalize_(self, x):
         """The rows of the float stream x take their own norm, in place."""
-        return ops.layer_norm(x, self.weight, self.eps, x)
+        return ops.layer_norm(x, self.weight, self.eps, x, bias=self.bias)
 
 
 register_part("norm", "rms_norm", RMSNorm)

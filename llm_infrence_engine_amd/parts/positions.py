@@ -7,6 +7,8 @@ the store of k and v into the cache pages.
 """
 from __future__ import annotations
 
+import math
+
 import torch
 
 from ..kernels import linear, ops
@@ -121,6 +123,67 @@ class QKNormTemperature(PositionEncoding):
                           kv.v_pages if store else None, bool(store and kv.v_transposed))
 
 
+def scaled_frequencies(dims: int, base: float, scaling=None) -> torch.Tensor:
+    """f_i = base^(-2 i / dims) for i < dims / 2, in double.  ``scaling`` {"factor", "low", "high", "original"} stretches
+    the long waves: with a wavelength l = 2 pi / f below original / high, f stays; above original / low, f / factor; in
+    between, with s = (original / l - low) / (high - low), the blend (1 - s) f / factor + s f."""
+    i = torch.arange(0, dims // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / max(1, dims))
+    if scaling is None:
+        return f
+    factor, low, high, original = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
+    if high == low:
+        raise ValueError("frequency scaling needs high != low")
+    wave = 2.0 * math.pi / f
+    s = (original / wave - low) / (high - low)
+    blended = (1.0 - s) * f / factor + s * f
+    return torch.where(wave < original / high, f, torch.where(wave > original / low, f / factor, blended))
+
+
+class QKNormRotaryHalf(PositionEncoding):
+    """Heads that are normalised and then rotated.  Every query and key head is divided by its root mean square (eps inside
+    the root) and, with ``weighted``, multiplied by a weight of its kind (``q_norm_name`` / ``k_norm_name`` [head_dim], shared
+    by the heads); then, with ``dims`` > 0, entry i and entry i + dims / 2 of the head's first ``dims`` entries turn by
+    position * f_i (``scaled_frequencies``); the rest pass.  Keys and values may differ in size.  Norm, angles, sines and
+    cosines are float; one kernel also stores k and v into the pages."""
+
+    takes_value_dim = True
+
+    def __init__(self, prefix: str, head_dim: int, eps: float, weighted: bool = True, dims: int = 0, base: float = 10000.0,
+                 scaling=None, q_norm_name: str = "q.norm", k_norm_name: str = "k.norm"):
+        if dims % 2 or not 0 <= dims <= head_dim:
+            raise ValueError(f"{dims} rotated entries must be even and within the head's {head_dim}")
+        self.prefix, self.head_dim, self.eps, self.weighted = prefix, head_dim, float(eps), bool(weighted)
+        self.dims, self.base = int(dims), float(base)
+        self.scaling = dict(scaling) if scaling is not None else None
+        self.q_norm_name, self.k_norm_name = q_norm_name, k_norm_name
+        self.q_weight = self.k_weight = self.inv_freq = None
+
+    def tensor_specs(self):
+        if not self.weighted:
+            return []
+        from ..weights.spec import TensorSpec
+
+        return [TensorSpec(self.prefix + self.q_norm_name, (self.head_dim,), "norm"),
+                TensorSpec(self.prefix + self.k_norm_name, (self.head_dim,), "norm")]
+
+    def load(self, get, rt):
+        self.rt = rt
+        if self.weighted:
+            self.q_weight, self.k_weight = (get(s) for s in self.tensor_specs())
+        if self.dims:
+            self.inv_freq = scaled_frequencies(self.dims, self.base, self.scaling).to(torch.float32).to(rt.device)
+
+    def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, kv, value_dim=None):
+        store = kv is not None and kv.store
+        ops.qk_norm_store(qkv, num_heads, num_kv_heads, head_dim, head_dim if value_dim is None else value_dim,
+                          self.q_weight, self.k_weight, self.eps, ctx.positions, 0.0, 1,
+                          kv.slot_mapping if store else None, kv.k_pages if store else None,
+                          kv.v_pages if store else None, bool(store and kv.v_transposed), unit_norm=True,
+                          inv_freq=self.inv_freq, rot_dim=self.dims)
+
+
+register_part("position", "qk_norm_rotary_half", QKNormRotaryHalf)
 register_part("position", "qk_norm_temperature", QKNormTemperature)
 register_part("position", "rotary_half", RotaryHalf)
 register_part("position", "rotary_pairs", RotaryPairs)
