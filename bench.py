@@ -26,7 +26,9 @@ random weights, bfloat16); one JSON line, ``sizes[width][design]``.  ``--design 
 decoder (selective scan, delta rule with a decay per head, two attention layers with a sink; every second feed-forward
 routed over sixteen experts) beside Gemadra and Qwen2, ``--design kuvazen`` for the Kuvazen decoder (minGRU and
 window-plus-pooled-blocks attention in turn, dense clamped and routed gated feed-forwards, a side input per layer) beside
-Gidurax and Qwen2.
+Gidurax and Qwen2, ``--design silizen`` for the Silizen decoder (attention beside gated linear attention, windowed attention
+beside the delta rule, a token-shifted recurrence; one norm per layer, feed-forwards gated with the tanh gelu) beside
+Gemadra and Qwen2.
 """
 from __future__ import annotations
 
@@ -273,7 +275,8 @@ def run_design(eng, a):
 
     from llm_infrence_engine_amd.config import config_from_dict, preset
 
-    beside = {"gemadra": ["qwen2"], "gidurax": ["gemadra", "qwen2"], "kuvazen": ["gidurax", "qwen2"]}[a.design]
+    beside = {"gemadra": ["qwen2"], "gidurax": ["gemadra", "qwen2"], "kuvazen": ["gidurax", "qwen2"],
+              "silizen": ["gemadra", "qwen2"]}[a.design]
     out = {"design": a.design, "beside": ",".join(beside), "layers": a.design_layers, "dtype": "bf16", "data": "synthetic",
            "prefill_tokens": PREFILL_TOKENS, "prompt_len": a.prompt_len, "sizes": {}}
     for size in a.design_sizes.split(","):
@@ -313,14 +316,14 @@ def run_design(eng, a):
 
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
-    ap.add_argument("--design", choices=["gemadra", "gidurax", "kuvazen"], default=None,
+    ap.add_argument("--design", choices=["gemadra", "gidurax", "kuvazen", "silizen"], default=None,
                     help="measure this design beside the closest existing ones (Gemadra beside Qwen2; Gidurax beside "
-                         "Gemadra and Qwen2; Kuvazen beside Gidurax and Qwen2) at equal sizes instead of the default workload")
+                         "Gemadra and Qwen2; Kuvazen beside Gidurax and Qwen2; Silizen beside Gemadra and Qwen2) at equal sizes instead of the default workload")
     ap.add_argument("--design-layers", type=int, default=4, help="layers of each model in a --design run")
     ap.add_argument("--design-sizes", default="0.5b,7b", help="widths of a --design run (0.5b, 7b)")
     ap.add_argument("--design-part", choices=["all", "prefill", "decode"], default="all",
                     help="a --design run's prompt step or its decode steps alone (for profiles)")
-    ap.add_argument("--design-only", choices=["gemadra", "gidurax", "kuvazen", "qwen2"], default=None,
+    ap.add_argument("--design-only", choices=["gemadra", "gidurax", "kuvazen", "silizen", "qwen2"], default=None,
                     help="one of the two models of a --design run alone (for profiles)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)

@@ -95,6 +95,33 @@ PRESETS["kuvazen-7b"] = _kuvazen(
      "rot": {"base": 10000.0, "dims": 128}}, (6336, 16, 3), 256, vocab=152064)
 
 
+def _silizen(width, ff, layers, attention, linear, delta, wkv_, window, rank, vocab=151936):
+    """``layers`` layers in the order parallel, parallel_2, wkv, parallel, ...; every layer with the dense gated
+    feed-forward; no looped stretch."""
+    rotated = dict(attention, softcap=30.0, rot={"base": 1000000.0, "dims": attention["dim"] // 2,
+                                                 "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}})
+    kinds = [("parallel", {"left": rotated, "right": dict(linear, tau=16.0, decay_rank=rank), "left_scale": 0.5, "right_scale": 0.5}),
+             ("parallel_2", {"left": dict(attention, mask={"size": window}), "right": dict(delta, conv=4, decay_rank=rank, gate_rank=rank)}),
+             ("wkv", dict(wkv_, decay_rank=rank))]
+    order = [0, 1, 2, 0]
+    import copy
+
+    return {"architecture": "Silizen", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "logit_scale": 1.0,
+            "layers": [{"type": kinds[order[i % 4]][0], "mixer": copy.deepcopy(kinds[order[i % 4]][1]),
+                        "mlp": {"kind": "dense", "ff": ff}} for i in range(layers)]}
+
+
+# Silizen at the same widths: attention of the Qwen2 shapes' heads beside a recurrence of the model's width, gated dense
+# feed-forwards of the Qwen2 shapes' size, a window of 1,024 tokens in the windowed attention
+PRESETS["silizen-0.5b"] = _silizen(
+    896, 4864, 24, {"heads": 14, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 64 ** -0.5},
+    {"heads": 7, "dim": 64, "vdim": 128}, {"heads": 14, "kv_heads": 7, "dim": 64, "vdim": 64}, {"heads": 14, "dim": 64}, 1024, 64)
+PRESETS["silizen-7b"] = _silizen(
+    3584, 18944, 28, {"heads": 28, "kv_heads": 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5},
+    {"heads": 28, "dim": 64, "vdim": 128}, {"heads": 28, "kv_heads": 14, "dim": 128, "vdim": 128}, {"heads": 28, "dim": 128}, 1024,
+    128, vocab=152064)
+
+
 def preset(name: str) -> dict:
     if name not in PRESETS:
         raise KeyError(f"no preset {name!r}; there are {', '.join(sorted(PRESETS))}")

@@ -116,7 +116,8 @@ int ms_paged_attention_mfma(const void* q, long long q_stride, const void* k_pag
                             const int* block_table, int table_stride, const int* table_rows, const int* q_start,
                             const int* context_lens, void* out, long long out_stride, int n_requests, int n_tokens,
                             int max_q_len, int num_heads, int num_kv_heads, int head_dim, int page_size, float scale,
-                            int window, const float* sink, hipStream_t stream);
+                            int window, const float* sink, float softcap, const float* slopes, const void* gate,
+                            long long gate_stride, float out_scale, hipStream_t stream);
 
 int ms_paged_attention_mfma_decode(const void* q, long long q_stride, const void* k_pages, const void* vt_pages,
                                    const int* block_table, int table_stride, const int* table_rows,
@@ -124,7 +125,8 @@ int ms_paged_attention_mfma_decode(const void* q, long long q_stride, const void
                                    void* part_o,
                                    void* part_ml, int n_requests, int num_heads, int num_kv_heads, int head_dim,
                                    int page_size, float scale, int window, int min_blocks, int n_splits,
-                                   const float* sink, hipStream_t stream);
+                                   const float* sink, float softcap, const float* slopes, const void* gate,
+                                   long long gate_stride, float out_scale, hipStream_t stream);
 
 int ms_argmax(const float* logits, long long ld, int n_rows, int vocab, float* scratch_val, int* scratch_idx,
               int n_chunks, int* out, hipStream_t stream);
@@ -305,7 +307,8 @@ int ms_gelu_tanh_glu(const void* gu, long long in_stride, void* out, long long o
 int ms_decay_recurrence(const void* q, const void* k, const void* v, long long q_stride, long long k_stride,
                         long long v_stride, const float* z, const float* z_bias, int decay_kind, float inv_tau,
                         const float* bonus, float q_scale, float* state, const int* q_start, const int* state_slots,
-                        float* out, int n_requests, int heads, int dim, int vdim, int dtype, hipStream_t stream);
+                        float* out, int n_requests, int heads, int dim, int vdim, int stretch, int max_stretches,
+                        float* pair_a, float* pair_b, int dtype, hipStream_t stream);
 int ms_token_shift(const void* h, long long h_stride, const float* mu, void* state, const int* token_req,
                    const int* q_start, const int* state_slots, const int* n_live_tokens, void* out, int n_tokens,
                    int n_requests, int width, int n_mixes, int dtype, hipStream_t stream);

@@ -114,15 +114,37 @@ __device__ __forceinline__ void load_values(ValueBlock<CT>& b, const bf16* __res
 // but only D / VS of the output's dims, so it reads all keys and 1 / VS of the values.  A compute unit draws
 // its data at a small fraction of the chip's rate, so when a step has fewer tiles than the chip has units this
 // shortens the longest chain without a second kernel; the blocks write disjoint dims and share nothing.
-template <int D, int NT, int WAVES, bool SPLIT, int VS, bool SINK>
-__global__ void __launch_bounds__(WAVES * MS_WAVE, (NT > 1 ? 2 : 1))
+// EXTRA: the scores are changed on their way into the softmax: a scaled score x becomes cap * tanh(x / cap) (cap > 0),
+// then slope * (the key's distance from the query) is taken off it, one slope per query head; at the end every head's
+// result is multiplied by out_scale and by the sigmoid of a gate, one number per token and head.  Such scores are kept
+// in log2 units from the start, and the block's maxima are those of the changed scores.
+struct AttnExtras {
+  float scale;               // of the raw scores, natural units
+  float cap;                 // 0: no cap
+  float exp_arg;             // 2 log2(e) / cap: tanh(x / cap) = 1 - 2 / (2^(x exp_arg) + 1)
+  const float* slopes;       // [nh] or null
+  const bf16* gate;          // [N, >= nh] or null
+  size_t gate_stride;
+  float out_scale;
+};
+
+// The variants that change their scores need more registers than two wide tiles to a SIMD leave: a wide tile of theirs
+// has the SIMD to itself.  Narrow tiles over sixteen waves (128 registers a lane) and the narrow tile of the largest
+// head over eight have no such variant, nor have wide tiles over eight waves; the launcher picks a neighbour.
+template <int D, int NT, int WAVES, int VS>
+constexpr bool extra_variant() {
+  return !(NT == 1 && WAVES == 16) && !(D == 128 && NT == 1 && WAVES == 8 && VS == 1) && !(NT > 1 && WAVES == 8);
+}
+
+template <int D, int NT, int WAVES, bool SPLIT, int VS, bool SINK, bool EXTRA = false>
+__global__ void __launch_bounds__(WAVES * MS_WAVE, (NT > 1 && !EXTRA ? 2 : 1))
 attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* __restrict__ k_pages,
                       const bf16* __restrict__ vt_pages, const int* __restrict__ block_table, int table_stride,
                       const int* __restrict__ table_rows, const int* __restrict__ q_start,
                       const int* __restrict__ context_lens, bf16* __restrict__ out, size_t out_stride,
                       float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv, int page_size,
                       int page_shift, float scale_log2e, int window, int min_blocks, int n_splits,
-                      const float* __restrict__ sink) {
+                      const float* __restrict__ sink, AttnExtras ex = AttnExtras()) {
   // SPLIT: min_blocks and n_splits say how a request's key blocks are spread.  Else min_blocks != 0 asks for
   // the order of tiles in which a long tile's companion on its CU is a short one (see below), and n_splits is
   // the number of requests whose tiles the grid's second dimension runs over (0: one tile to a request)
@@ -227,6 +249,11 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
 
   // this lane's columns
   int pos[NT];   // -1: an idle column (sees no key; its result is not written)
+  float slope[EXTRA ? NT : 1];
+  const float sl2 = EXTRA ? 1.0f : scale_log2e;   // what turns a kept score into log2 units
+  // the fields the loop reads, as scalars of their own (the struct itself stays in the kernel's arguments)
+  const float ex_scale = ex.scale, ex_cap = ex.cap, ex_arg = ex.exp_arg;
+  const float* const ex_slopes = ex.slopes;
   bf16x8 qv[NT][D / 32];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
@@ -234,6 +261,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
     const int cc = min(c, ncols - 1);
     const int tok = q0 + cc / rep, head = g * rep + cc % rep;
     pos[t] = c < ncols ? start_pos + cc / rep : -1;
+    if (EXTRA) slope[t] = ex_slopes ? ex_slopes[head] : 0.f;
     const bf16* qp = q + (size_t)tok * q_stride + (size_t)head * D + kq * 8;
 #pragma unroll
     for (int s = 0; s < D / 32; ++s) qv[t][s] = *reinterpret_cast<const bf16x8*>(qp + s * 32);
@@ -262,7 +290,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   // A sink is one more term of the denominator with no key and no value: the running softmax of one wave (the first
   // wave of the block, of the first split) starts as if it had already seen a key with that score, unscaled, and a
   // value of zero.  Everything after (moving the reference, merging waves and splits) treats it as any other term.
-  if (SINK && wave == 0 && (!SPLIT || bx == 0)) {
+  if (SINK && sink && wave == 0 && (!SPLIT || bx == 0)) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int cc = min(c0 + t * 16 + col16, ncols - 1);
@@ -275,7 +303,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   // A narrow tile (decode) has registers to spare and few waves to hide a wait behind: it fetches the next
   // block's values early, together with its keys.  A wide tile fetches values at the top of the pass that
   // uses them (the score products and the softmax run meanwhile, and so does the SIMD's other wave).
-  constexpr bool VALUES_EARLY = NT == 1;
+  constexpr bool VALUES_EARLY = NT == 1 && !EXTRA;   // (changed scores need the registers)
   KeyBlock<D> buf_k[2];
   ValueBlock<CT> buf_v[2];
   BlockPlace buf_at[2];
@@ -325,6 +353,22 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
         for (int ks = 0; ks < D / 32; ++ks) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur_k.k[u][ks], qv[t][ks], acc, 0, 0, 0);
         s[u][t] = acc;
       }
+
+    if (EXTRA) {
+      // slope * (pos - key) = slope * (pos - base - 4 kq) - slope * (16 u + i): one product per column, then constants
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const float off = -slope[t] * (float)(pos[t] - base - kq * 4);
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float x = s[u][t][i] * ex_scale;
+            if (ex_cap > 0.f) x = fmaf(-2.0f * ex_cap, __builtin_amdgcn_rcpf(fast_exp2(x * ex_arg) + 1.0f), ex_cap);
+            s[u][t][i] = (x + fmaf(slope[t], (float)(u * 16 + i), off)) * 1.4426950408889634f;
+          }
+      }
+    }
 
     // values past the last visible key may be anything a reused page still holds: make them zero
     if (base + 31 > key_hi) {
@@ -377,7 +421,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
       float bm = bmax[t];
       bm = fmaxf(bm, __shfl_xor(bm, 16, MS_WAVE));
       bm = fmaxf(bm, __shfl_xor(bm, 32, MS_WAVE));
-      bm *= scale_log2e;
+      bm *= sl2;
       // m is the reference that the exponents are taken against, not necessarily the maximum: it follows the
       // maximum only when that has run ahead by more than REF_SLACK (a factor 2^REF_SLACK in the terms, far
       // inside float's range), so that the accumulators are rescaled rarely.  Any reference gives the same
@@ -405,7 +449,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
       for (int u = 0; u < 2; ++u)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float e = fast_exp2(fmaf(s[u][t][i], scale_log2e, -m_safe[t]));
+          const float e = fast_exp2(fmaf(s[u][t][i], sl2, -m_safe[t]));
           if (!SUMS_BY_MATRIX) lvec[t] += e;
           p[t][u * 4 + i] = (__bf16)e;
         }
@@ -480,7 +524,12 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
       for (int c = 0; c < CT; ++c) *reinterpret_cast<f32x4*>(po + c * 16) = o[c][t];
       if (kq == 0) { part_ml[slot * 2] = m[t]; part_ml[slot * 2 + 1] = lt; }
     } else {
-      const float inv = 1.0f / lt;
+      float inv = 1.0f / lt;
+      if (EXTRA) {
+        inv *= ex.out_scale;
+        if (ex.gate)
+          inv *= __builtin_amdgcn_rcpf(1.0f + fast_exp2(-1.4426950408889634f * __bfloat162float(ex.gate[(size_t)tok * ex.gate_stride + head])));
+      }
       bf16* op = out + (size_t)tok * out_stride + (size_t)head * D + dim0 + kq * 4;
 #pragma unroll
       for (int c = 0; c < CT; ++c) {
@@ -503,7 +552,7 @@ __global__ void __launch_bounds__(D < 64 ? 64 : D)
 attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                          const int* __restrict__ q_start, const int* __restrict__ context_lens,
                          bf16* __restrict__ out, size_t out_stride, int nh, int window, int min_blocks,
-                         int n_splits) {
+                         int n_splits, const bf16* __restrict__ gate, size_t gate_stride, float out_scale) {
   __shared__ float sm_m[COMBINE_MAX_SPLITS], sm_w[COMBINE_MAX_SPLITS];
   const int r = blockIdx.x / nh, h = blockIdx.x % nh;
   if (q_start[r + 1] == q_start[r]) return;   // a row that pads a captured batch: no token, nothing to write
@@ -528,7 +577,8 @@ attention_combine_kernel(const float* __restrict__ part_o, const float* __restri
   __syncthreads();
   float den = 0.f;
   for (int s = 0; s < used; ++s) den += sm_m[s];
-  const float inv = 1.0f / den;
+  float inv = out_scale / den;
+  if (gate) inv *= 1.0f / (1.0f + expf(-__bfloat162float(gate[(size_t)q_start[r] * gate_stride + h])));
   bf16* op = out + (size_t)q_start[r] * out_stride + (size_t)h * D;
   for (int d = t; d < D; d += blockDim.x) {
     float acc = 0.f;
@@ -551,7 +601,7 @@ template <int D, int NT, int WAVES, int VS>
 int launch_general(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, const int* table, int table_stride,
                    const int* table_rows, const int* q_start, const int* ctx, bf16* out, size_t out_stride,
                    int n_requests, int n_tokens, int max_q_len, int nh, int nkv, int page_size, float scale,
-                   int window, const float* sink, hipStream_t stream) {
+                   int window, const float* sink, const AttnExtras* extras, hipStream_t stream) {
   const int rep = nh / nkv;
   const long long per_request = ((long long)max_q_len * rep + 16 * NT - 1) / (16 * NT);
   // every request may end in a partial tile; no step has more tiles than if each request were the longest
@@ -561,8 +611,15 @@ int launch_general(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt
   const int pair_order = tiles * VS * nkv <= 2LL * ms_compute_units() ? 1 : 0;
   const int scan = per_request == 1 ? 0 : n_requests;   // one tile to a request: the tile's index is the request's
   dim3 grid(nkv, (unsigned)tiles, VS), block(WAVES * MS_WAVE);
-  if constexpr (D == 64 && NT == 4) {     // no variant with a sink at this shape (its registers are spent)
-    if (sink) return MS_UNSUPPORTED;
+  if constexpr (D == 64 && NT == 4) {     // no variant with a sink or changed scores at this shape (its registers are spent)
+    if (sink || extras) return MS_UNSUPPORTED;
+  } else if (extras) {
+    if constexpr (extra_variant<D, NT, WAVES, VS>()) {
+      attention_mfma_kernel<D, NT, WAVES, false, VS, true, true><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, table_rows, q_start, ctx, out, out_stride, nullptr, nullptr, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, pair_order, scan, sink, *extras);
+      return ms_launch_status();
+    } else {
+      return MS_UNSUPPORTED;
+    }
   } else if (sink) {
     attention_mfma_kernel<D, NT, WAVES, false, VS, true><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, table_rows, q_start, ctx, out, out_stride, nullptr, nullptr, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, pair_order, scan, sink);
     return ms_launch_status();
@@ -575,13 +632,15 @@ template <int D>
 int launch_split(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, const int* table, int table_stride,
                  const int* table_rows, const int* q_start, const int* ctx, bf16* out, size_t out_stride, float* part_o, float* part_ml,
                  int n_requests, int nh, int nkv, int page_size, float scale, int window, int min_blocks,
-                 int n_splits, const float* sink, hipStream_t stream) {
+                 int n_splits, const float* sink, const AttnExtras* extras, hipStream_t stream) {
   dim3 grid(n_splits, nkv, n_requests), block(4 * MS_WAVE);
-  if (sink)
+  if (extras)
+    attention_mfma_kernel<D, 1, 4, true, 1, true, true><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, table_rows, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, min_blocks, n_splits, sink, *extras);
+  else if (sink)
     attention_mfma_kernel<D, 1, 4, true, 1, true><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, table_rows, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, min_blocks, n_splits, sink);
   else
     attention_mfma_kernel<D, 1, 4, true, 1, false><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, table_rows, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, min_blocks, n_splits, nullptr);
-  attention_combine_kernel<D><<<dim3(n_requests * nh), dim3(D < 64 ? 64 : D), 0, stream>>>(part_o, part_ml, q_start, ctx, out, out_stride, nh, window, min_blocks, n_splits);
+  attention_combine_kernel<D><<<dim3(n_requests * nh), dim3(D < 64 ? 64 : D), 0, stream>>>(part_o, part_ml, q_start, ctx, out, out_stride, nh, window, min_blocks, n_splits, extras ? extras->gate : nullptr, extras ? extras->gate_stride : 0, extras ? extras->out_scale : 1.0f);
   return ms_launch_status();
 }
 
@@ -612,14 +671,19 @@ extern "C" int ms_paged_attention_mfma(const void* q, long long q_stride, const 
                                        const int* q_start, const int* context_lens, void* out, long long out_stride,
                                        int n_requests, int n_tokens, int max_q_len, int num_heads, int num_kv_heads,
                                        int head_dim, int page_size, float scale, int window, const float* sink,
-                                       hipStream_t stream) {
+                                       float softcap, const float* slopes, const void* gate, long long gate_stride,
+                                       float out_scale, hipStream_t stream) {
   if (n_requests <= 0 || max_q_len <= 0 || n_tokens <= 0) return MS_OK;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || table_stride <= 0) return MS_BAD_ARG;
   if (!(scale > 0.f)) return MS_BAD_ARG;   // maxima are taken of the raw scores
   if (!ms_attention_mfma_supported(head_dim, page_size)) return MS_UNSUPPORTED;
   if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q % 16) || ((uintptr_t)out % 8)) return MS_UNSUPPORTED;
   if (n_requests > 65535 || num_kv_heads > 65535) return MS_UNSUPPORTED;
-#define GO(D, NT, WV, VS) return launch_general<D, NT, WV, VS>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, table_rows, q_start, context_lens, (bf16*)out, out_stride, n_requests, n_tokens, max_q_len, num_heads, num_kv_heads, page_size, scale, window, sink, stream)
+  const bool changed = softcap > 0.f || slopes != nullptr || gate != nullptr || out_scale != 1.0f;
+  const AttnExtras ex = {scale, softcap > 0.f ? softcap : 0.f, softcap > 0.f ? 2.0f * 1.4426950408889634f / softcap : 0.f,
+                         slopes, (const bf16*)gate, (size_t)gate_stride, out_scale};
+  const AttnExtras* extras = changed ? &ex : nullptr;
+#define GO(D, NT, WV, VS) return launch_general<D, NT, WV, VS>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, table_rows, q_start, context_lens, (bf16*)out, out_stride, n_requests, n_tokens, max_q_len, num_heads, num_kv_heads, page_size, scale, window, sink, extras, stream)
   // Tile width (NT * 16 columns) and waves over a tile's keys.  Few columns (a decode step): one narrow tile
   // per request and many waves over its keys.
   const int cols = max_q_len * (num_heads / num_kv_heads);
@@ -639,7 +703,11 @@ extern "C" int ms_paged_attention_mfma(const void* q, long long q_stride, const 
     if (head_dim == 128 && tiles >= 2LL * cus) waves = 4;
   }
   // with a sink the widest tile at head size 64 has no register left for the softmax's other starting point
-  if (sink != nullptr && head_dim == 64 && nt == 4) nt = 2;
+  if ((sink != nullptr || changed) && head_dim == 64 && nt == 4) nt = 2;
+  if (changed && nt == 1) {     // the variants with changed scores: eight waves over a narrow tile's keys, four at 128 dims
+    if (head_dim == 32) vs = 1;
+    waves = head_dim == 128 && vs == 1 ? 4 : 8;
+  }
   if (g_force_nt) { nt = g_force_nt; waves = g_force_waves; }
   if (g_force_vs) vs = g_force_vs;
   if (nt > 1) vs = 1;
@@ -668,7 +736,8 @@ extern "C" int ms_paged_attention_mfma_decode(const void* q, long long q_stride,
                                               long long out_stride, void* part_o, void* part_ml, int n_requests,
                                               int num_heads, int num_kv_heads, int head_dim, int page_size,
                                               float scale, int window, int min_blocks, int n_splits, const float* sink,
-                                              hipStream_t stream) {
+                                              float softcap, const float* slopes, const void* gate, long long gate_stride,
+                                              float out_scale, hipStream_t stream) {
   if (n_requests <= 0) return MS_OK;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || table_stride <= 0) return MS_BAD_ARG;
   if (num_heads / num_kv_heads > 16) return MS_UNSUPPORTED;
@@ -677,7 +746,11 @@ extern "C" int ms_paged_attention_mfma_decode(const void* q, long long q_stride,
   if (min_blocks <= 0 || n_splits <= 0 || n_splits > COMBINE_MAX_SPLITS) return MS_BAD_ARG;
   if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q % 16) || ((uintptr_t)out % 8) || ((uintptr_t)part_o % 16)) return MS_UNSUPPORTED;
   if (n_requests > 65535 || num_kv_heads > 65535) return MS_UNSUPPORTED;
-#define GO(D) return launch_split<D>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, table_rows, q_start, context_lens, (bf16*)out, out_stride, (float*)part_o, (float*)part_ml, n_requests, num_heads, num_kv_heads, page_size, scale, window, min_blocks, n_splits, sink, stream)
+  const bool changed = softcap > 0.f || slopes != nullptr || gate != nullptr || out_scale != 1.0f;
+  const AttnExtras ex = {scale, softcap > 0.f ? softcap : 0.f, softcap > 0.f ? 2.0f * 1.4426950408889634f / softcap : 0.f,
+                         slopes, (const bf16*)gate, (size_t)gate_stride, out_scale};
+  const AttnExtras* extras = changed ? &ex : nullptr;
+#define GO(D) return launch_split<D>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, table_rows, q_start, context_lens, (bf16*)out, out_stride, (float*)part_o, (float*)part_ml, n_requests, num_heads, num_kv_heads, page_size, scale, window, min_blocks, n_splits, sink, extras, stream)
   if (head_dim == 32) GO(32);
   if (head_dim == 64) GO(64);
   GO(128);

@@ -40,33 +40,73 @@ constexpr int DPT = 16;           // rows of a column a lane holds
 // Column j of S depends on no other column: LPC neighbouring lanes hold it (DPT rows each) for the whole portion.  A
 // block owns REC_THREADS / LPC columns of one (request, head).  Tokens are staged a chunk at a time (q scaled, k, the
 // decay worked out, v) as floats in LDS, then walked in order.
-template <typename T, int LPC, bool BONUS>
+//
+// A long portion is spread over blocks (MODE 1, then MODE 2; MODE 0 walks the whole portion in one block): the recurrence
+// is linear in S, so a stretch of `stretch` tokens maps the state it starts from to diag(A) S + B, A the product of its
+// decays and B what it leaves when started from zero.  MODE 1: every stretch but a portion's last walks from zero and
+// leaves A and B in scratch; the last one's block puts a copy of the request's state there instead (its own pair is never
+// asked for), so that the second launch, whose last stretch overwrites the state, reads the state from the copy whenever
+// its blocks run.  MODE 2: every stretch folds the pairs of the stretches before it onto that copy, in order, walks from
+// there and writes the read-outs; the last one stores the state.  blockIdx.z = request * stretches
+// a request may have + the stretch's index.
+template <typename T, int LPC, bool BONUS, int MODE>
 __global__ void __launch_bounds__(REC_THREADS)
 decay_recurrence_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, size_t q_stride,
                         size_t k_stride, size_t v_stride, const float* __restrict__ z, const float* __restrict__ z_bias,
                         int decay_kind, float inv_tau, const float* __restrict__ bonus, float q_scale,
                         float* __restrict__ state, const int* __restrict__ q_start, const int* __restrict__ state_slots,
-                        float* __restrict__ out, int H, int D, int E) {
+                        float* __restrict__ out, int H, int D, int E, int stretch, int max_stretches,
+                        float* __restrict__ pair_a, float* __restrict__ pair_b) {
   constexpr int Dp = DPT * LPC, COLS = REC_THREADS / LPC;
   __shared__ __align__(16) float qs[REC_CHUNK * Dp];
   __shared__ __align__(16) float ks[REC_CHUNK * Dp];
   __shared__ __align__(16) float ws[REC_CHUNK * Dp];
   __shared__ float vs[REC_CHUNK * COLS];
-  const int r = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * COLS;
+  const int r = MODE == 0 ? blockIdx.z : blockIdx.z / max_stretches, h = blockIdx.y, col0 = blockIdx.x * COLS;
+  const int piece = MODE == 0 ? 0 : blockIdx.z - r * max_stretches;
   const int s0 = q_start[r], L = q_start[r + 1] - s0;
   if (L <= 0) return;
+  const int t_begin = MODE == 0 ? 0 : piece * stretch;
+  const int t_end = MODE == 0 ? L : min(L, t_begin + stretch);
+  if (t_begin >= L) return;
   const int tid = threadIdx.x, part = tid % LPC, my = tid / LPC, col = col0 + my;
   const bool live = col < E;
   float* Sg = state + (((size_t)state_slots[r] * H + h) * D) * E;
-  float S[DPT], U[DPT];
+  float S[DPT], U[DPT], A[MODE == 1 ? DPT : 1];
 #pragma unroll
   for (int ii = 0; ii < DPT; ++ii) {
     const int i = part * DPT + ii;
-    S[ii] = (live && i < D) ? Sg[(size_t)i * E + col] : 0.f;
+    S[ii] = (MODE == 0 && live && i < D) ? Sg[(size_t)i * E + col] : 0.f;
     U[ii] = (BONUS && i < D) ? bonus[(size_t)h * D + i] : 0.f;
+    if (MODE == 1) A[ii] = 1.f;
   }
-  for (int c0 = 0; c0 < L; c0 += REC_CHUNK) {
-    const int cn = min(REC_CHUNK, L - c0);
+  if (MODE == 1 && t_end == L) {      // a portion's last stretch: the state's copy
+    const size_t at = ((size_t)r * max_stretches + piece) * H + h;
+#pragma unroll
+    for (int ii = 0; ii < DPT; ++ii) {
+      const int i = part * DPT + ii;
+      if (live && i < D) pair_b[(at * D + i) * E + col] = Sg[(size_t)i * E + col];
+    }
+    return;
+  }
+  if (MODE == 2) {
+    const size_t copy = ((size_t)r * max_stretches + (L - 1) / stretch) * H + h;
+#pragma unroll
+    for (int ii = 0; ii < DPT; ++ii) {
+      const int i = part * DPT + ii;
+      if (live && i < D) S[ii] = pair_b[(copy * D + i) * E + col];
+    }
+    for (int c = 0; c < piece; ++c) {
+      const size_t at = ((size_t)r * max_stretches + c) * H + h;
+#pragma unroll
+      for (int ii = 0; ii < DPT; ++ii) {
+        const int i = part * DPT + ii;
+        if (live && i < D) S[ii] = fmaf(pair_a[at * D + i], S[ii], pair_b[(at * D + i) * E + col]);
+      }
+    }
+  }
+  for (int c0 = t_begin; c0 < t_end; c0 += REC_CHUNK) {
+    const int cn = min(REC_CHUNK, t_end - c0);
     __syncthreads();      // the chunk before has been walked
     for (int e = tid; e < cn * Dp; e += REC_THREADS) {
       const int t = e / Dp, i = e - t * Dp;
@@ -101,7 +141,10 @@ decay_recurrence_kernel(const T* __restrict__ q, const T* __restrict__ k, const 
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const float write = kk[j] * vt;
-          if (BONUS) {
+          if (MODE == 1) {
+            S[ii + j] = fmaf(ww[j], S[ii + j], write);
+            A[ii + j] *= ww[j];
+          } else if (BONUS) {
             o4[j] = fmaf(fmaf(U[ii + j], write, S[ii + j]), qq[j], o4[j]);
             S[ii + j] = fmaf(ww[j], S[ii + j], write);
           } else {
@@ -110,10 +153,23 @@ decay_recurrence_kernel(const T* __restrict__ q, const T* __restrict__ k, const 
           }
         }
       }
-      const float o = group_sum<LPC>((o4[0] + o4[1]) + (o4[2] + o4[3]));
-      if (live && part == 0) out[((size_t)(s0 + c0 + t) * H + h) * E + col] = o;
+      if (MODE != 1) {
+        const float o = group_sum<LPC>((o4[0] + o4[1]) + (o4[2] + o4[3]));
+        if (live && part == 0) out[((size_t)(s0 + c0 + t) * H + h) * E + col] = o;
+      }
     }
   }
+  if (MODE == 1) {
+    const size_t at = ((size_t)r * max_stretches + piece) * H + h;
+#pragma unroll
+    for (int ii = 0; ii < DPT; ++ii) {
+      const int i = part * DPT + ii;
+      if (live && i < D) pair_b[(at * D + i) * E + col] = S[ii];
+      if (blockIdx.x == 0 && my == 0 && i < D) pair_a[at * D + i] = A[ii];
+    }
+    return;
+  }
+  if (t_end < L) return;      // (MODE 2) only a portion's last stretch leaves the state
 #pragma unroll
   for (int ii = 0; ii < DPT; ++ii) {
     const int i = part * DPT + ii;
@@ -203,25 +259,35 @@ extern "C" int ms_tanh(void* x, long long total, int dtype, hipStream_t stream) 
 
 // q, k [N, >= heads * dim] and v [N, >= heads * vdim] of `dtype`, rows q_stride / k_stride / v_stride elements apart;
 // z float [N, heads * dim], z_bias (may be null) float [heads * dim]; bonus (may be null) float [heads * dim];
-// state float [slots, heads, dim, vdim]; out float [N, heads * vdim].
+// state float [slots, heads, dim, vdim]; out float [N, heads * vdim].  max_stretches > 1: every portion is cut into
+// stretches of `stretch` tokens (no portion has more than max_stretches of them) that run side by side in two launches;
+// pair_a float [n_requests, max_stretches, heads, dim] and pair_b float [n_requests, max_stretches, heads, dim, vdim] are
+// scratch.
 extern "C" int ms_decay_recurrence(const void* q, const void* k, const void* v, long long q_stride, long long k_stride,
                                    long long v_stride, const float* z, const float* z_bias, int decay_kind, float inv_tau,
                                    const float* bonus, float q_scale, float* state, const int* q_start,
                                    const int* state_slots, float* out, int n_requests, int heads, int dim, int vdim,
-                                   int dtype, hipStream_t stream) {
+                                   int stretch, int max_stretches, float* pair_a, float* pair_b, int dtype,
+                                   hipStream_t stream) {
   if (n_requests <= 0) return MS_OK;
   if (heads <= 0 || dim <= 0 || vdim <= 0 || (decay_kind != 0 && decay_kind != 1)) return MS_BAD_ARG;
   if (q_stride < (long long)heads * dim || k_stride < (long long)heads * dim || v_stride < (long long)heads * vdim)
     return MS_BAD_ARG;
   if (dim > DPT * 16) return MS_UNSUPPORTED;
+  const bool spread = max_stretches > 1;
+  if (spread && (stretch <= 0 || pair_a == nullptr || pair_b == nullptr)) return MS_BAD_ARG;
+  if (spread && (long long)n_requests * max_stretches > 65535) return MS_UNSUPPORTED;
   int lpc = 1;
   while (lpc * DPT < dim) lpc *= 2;
   const int cols = REC_THREADS / lpc;
-  dim3 grid((unsigned)((vdim + cols - 1) / cols), (unsigned)heads, (unsigned)n_requests), block(REC_THREADS);
+  dim3 grid((unsigned)((vdim + cols - 1) / cols), (unsigned)heads, (unsigned)(n_requests * (spread ? max_stretches : 1)));
+  dim3 block(REC_THREADS);
+#define LAUNCH4(T, LPC, B, MODE)                                                                                     \
+  decay_recurrence_kernel<T, LPC, B, MODE><<<grid, block, 0, stream>>>((const T*)q, (const T*)k, (const T*)v,        \
+      (size_t)q_stride, (size_t)k_stride, (size_t)v_stride, z, z_bias, decay_kind, inv_tau, bonus, q_scale, state, q_start, \
+      state_slots, out, heads, dim, vdim, stretch, max_stretches, pair_a, pair_b)
 #define LAUNCH3(T, LPC, B)                                                                                           \
-  decay_recurrence_kernel<T, LPC, B><<<grid, block, 0, stream>>>((const T*)q, (const T*)k, (const T*)v, (size_t)q_stride, \
-      (size_t)k_stride, (size_t)v_stride, z, z_bias, decay_kind, inv_tau, bonus, q_scale, state, q_start, state_slots, out, \
-      heads, dim, vdim)
+  do { if (spread) { LAUNCH4(T, LPC, B, 1); LAUNCH4(T, LPC, B, 2); } else LAUNCH4(T, LPC, B, 0); } while (0)
 #define LAUNCH2(T, LPC) do { if (bonus) LAUNCH3(T, LPC, true); else LAUNCH3(T, LPC, false); } while (0)
 #define LAUNCH(T)                                                                                                    \
   switch (lpc) {                                                                                                     \
@@ -237,6 +303,7 @@ extern "C" int ms_decay_recurrence(const void* q, const void* k, const void* v, 
 #undef LAUNCH
 #undef LAUNCH2
 #undef LAUNCH3
+#undef LAUNCH4
   return ms_launch_status();
 }
 

@@ -65,10 +65,11 @@ _SIGNATURES = {
                                    _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ll, _c_float, _c_int, _c_ptr],
     "ms_attention_mfma_supported": [_c_int, _c_int],
     "ms_paged_attention_mfma": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll,
-                                _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr, _c_ptr],
+                                _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr,
+                                _c_float, _c_ptr, _c_ptr, _c_ll, _c_float, _c_ptr],
     "ms_paged_attention_mfma_decode": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                        _c_ll, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
-                                       _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
+                                       _c_int, _c_int, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ll, _c_float, _c_ptr],
     "ms_argmax": [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr],
     "ms_sample": [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
                   _c_ptr],
@@ -81,7 +82,8 @@ _SIGNATURES = {
                            _c_int, _c_ptr],
     "ms_gelu_tanh_glu": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_ptr],
     "ms_decay_recurrence": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ll, _c_ll, _c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_float,
-                            _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+                            _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
+                            _c_int, _c_ptr],
     "ms_token_shift": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
                        _c_int, _c_ptr],
     "ms_pair_sum": [_c_ptr, _c_ptr, _c_float, _c_float, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
@@ -823,16 +825,25 @@ def attention_splits_keys(n_requests: int, num_kv_heads: int, group: int, max_q_
 def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, vt_pages: torch.Tensor, block_table: torch.Tensor,
                          q_start: torch.Tensor, context_lens: torch.Tensor, out: torch.Tensor, num_heads: int,
                          scale: float, max_q_len: int, max_context_len: int, window: Optional[int] = None,
-                         table_rows: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+                         table_rows: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None,
+                         softcap: float = 0.0, slopes: Optional[torch.Tensor] = None,
+                         gate: Optional[torch.Tensor] = None, out_scale: float = 1.0) -> torch.Tensor:
     """Matrix-core attention, bfloat16.  k_pages [P, nkv, page_size, d], vt_pages [P, nkv, d, page_size];
     request r owns tokens q_start[r]..q_start[r+1]-1, holds context_lens[r] keys after this step and has row
     ``table_rows[r]`` of ``block_table`` (row r without ``table_rows``).  ``max_q_len`` and ``max_context_len``
     are upper bounds; tokens from q_start[R] on belong to no request, a request may have no token.  A small
     batch of single tokens with long contexts also splits the keys over blocks (and combines).  ``sink`` float [nh]:
-    exp(sink[h]) joins the denominator of head h's softmax."""
+    exp(sink[h]) joins the denominator of head h's softmax.  ``softcap``, ``slopes``, ``gate`` and ``out_scale`` as in
+    ``paged_attention_generic``."""
     _check(k_pages, "k_pages", torch.bfloat16)
     if sink is not None:
         _check(sink, "sink", torch.float32, (num_heads,))
+    if slopes is not None:
+        _check(slopes, "slopes", torch.float32, (num_heads,))
+    gate_stride = _rows2d(gate, "gate", torch.bfloat16, num_heads) if gate is not None else 0
+    if gate is not None and gate.shape[0] != q.shape[0]:
+        raise ValueError("gate must have a row per token")
+    more = (float(softcap or 0.0), _ptr(slopes), _ptr(gate), gate_stride, float(out_scale))
     P, nkv, page_size, d = k_pages.shape
     _check(vt_pages, "vt_pages", torch.bfloat16, (P, nkv, d, page_size))
     _check(q, "q", torch.bfloat16, contiguous=False)
@@ -869,12 +880,12 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, vt_pages: torch
         _call("ms_paged_attention_mfma_decode", q.data_ptr(), q_stride, k_pages.data_ptr(), vt_pages.data_ptr(),
               block_table.data_ptr(), block_table.shape[1], _ptr(table_rows), q_start.data_ptr(), context_lens.data_ptr(),
               out.data_ptr(), num_heads * d, part_o.data_ptr(), part_ml.data_ptr(), R, num_heads, nkv, d, page_size, float(scale),
-              int(window or 0), MIN_BLOCKS_PER_SPLIT, n_splits, _ptr(sink), _stream())
+              int(window or 0), MIN_BLOCKS_PER_SPLIT, n_splits, _ptr(sink), *more, _stream())
     else:
         _call("ms_paged_attention_mfma", q.data_ptr(), q_stride, k_pages.data_ptr(), vt_pages.data_ptr(),
               block_table.data_ptr(), block_table.shape[1], _ptr(table_rows), q_start.data_ptr(), context_lens.data_ptr(),
               out.data_ptr(), num_heads * d, R, N, max_q_len, num_heads, nkv, d, page_size, float(scale), int(window or 0),
-              _ptr(sink), _stream())
+              _ptr(sink), *more, _stream())
     return out
 
 
@@ -921,8 +932,7 @@ def paged_attention(q: torch.Tensor, kv, ctx, out: torch.Tensor, num_heads: int,
     ``sink`` float [num_heads]: exp(sink[h]) joins the denominator of head h's softmax."""
     d, page_size = kv.k_pages.shape[3], kv.k_pages.shape[2]
     dv = kv.v_pages.shape[2] if kv.v_transposed else kv.v_pages.shape[3]
-    if dv != d or softcap or slopes is not None or gate is not None or out_scale != 1.0:
-        # capped scores, a distance penalty and an output gate are the generic kernel's
+    if dv != d:
         return paged_attention_generic(q, kv.k_pages, kv.v_pages, kv.block_table, ctx.token_req, ctx.positions, out,
                                        num_heads, scale, window, kv.v_transposed, kv.table_rows, ctx.n_live_tokens, sink,
                                        softcap, slopes, gate, out_scale)
@@ -933,9 +943,11 @@ def paged_attention(q: torch.Tensor, kv, ctx, out: torch.Tensor, num_heads: int,
     if (q.dtype == torch.bfloat16 and kv.v_transposed and attention_mfma_supported(d, page_size)
             and q.data_ptr() % 16 == 0 and (q.shape[0] == 1 or q.stride(0) % 8 == 0)):
         return paged_attention_mfma(q, kv.k_pages, kv.v_pages, kv.block_table, ctx.q_start, ctx.context_lens, out,
-                                    num_heads, scale, ctx.max_q_len, ctx.max_context_len, window, kv.table_rows, sink)
+                                    num_heads, scale, ctx.max_q_len, ctx.max_context_len, window, kv.table_rows, sink,
+                                    softcap, slopes, gate, out_scale)
     return paged_attention_generic(q, kv.k_pages, kv.v_pages, kv.block_table, ctx.token_req, ctx.positions, out,
-                                   num_heads, scale, window, kv.v_transposed, kv.table_rows, ctx.n_live_tokens, sink)
+                                   num_heads, scale, window, kv.v_transposed, kv.table_rows, ctx.n_live_tokens, sink,
+                                   softcap, slopes, gate, out_scale)
 
 
 # ------------------------------------------------------------------------------------------------ state-carrying mixers
@@ -1033,6 +1045,9 @@ def gated_head_norm(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, o
 
 
 DECAY_SIGMOID_ROOT, DECAY_DOUBLE_EXP = 0, 1
+RECURRENCE_STRETCH = 128             # tokens of a long portion that one block walks when the portion is spread over blocks
+RECURRENCE_SPREAD_FROM = 256         # the portion length from which that pays
+RECURRENCE_SCRATCH_BYTES = 1 << 29   # the most scratch a spread step may take
 
 
 def decay_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor, z_bias: Optional[torch.Tensor],
@@ -1043,7 +1058,9 @@ def decay_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch
     with ``bonus`` u float [heads * dim] the read comes first and weights the current token:
     o = (S + diag(u) k v^T)^T (q_scale q), then the write.  The decay is made from z float [N, heads * dim] (+ ``z_bias``
     float [heads * dim]): DECAY_SIGMOID_ROOT: w = sigmoid(z)^(1 / tau); DECAY_DOUBLE_EXP: w = exp(-exp(z)).  q, k
-    [N, heads * dim] and v [N, heads * vdim] may be row slices; out float [N, heads * vdim]."""
+    [N, heads * dim] and v [N, heads * vdim] may be row slices; out float [N, heads * vdim].  A step with long portions
+    (``ctx.max_q_len``, an upper bound) cuts them into stretches that run side by side and are joined through the
+    recurrence's linearity, in two launches; the float sums then associate differently, within rounding."""
     N = q.shape[0]
     sq = _rows2d(q, "q", None, heads * dim)
     sk = _rows2d(k, "k", q.dtype, heads * dim)
@@ -1064,9 +1081,19 @@ def decay_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch
     R = ctx.num_requests
     _check(ctx.q_start, "q_start", torch.int32, (R + 1,))
     _check(ctx.state_slots, "state_slots", torch.int32, (R,))
+    longest = min(int(getattr(ctx, "max_q_len", 0) or 0), N)
+    stretches, pair_a, pair_b = 1, None, None
+    if longest >= RECURRENCE_SPREAD_FROM:
+        stretches = -(-longest // RECURRENCE_STRETCH)
+        if R * stretches > 65535 or 4 * R * stretches * heads * dim * (vdim + 1) > RECURRENCE_SCRATCH_BYTES:
+            stretches = 1
+        else:
+            pair_a = torch.empty((R, stretches, heads, dim), dtype=torch.float32, device=q.device)
+            pair_b = torch.empty((R, stretches, heads, dim, vdim), dtype=torch.float32, device=q.device)
     _call("ms_decay_recurrence", q.data_ptr(), k.data_ptr(), v.data_ptr(), sq, sk, sv, z.data_ptr(), _ptr(z_bias), int(decay),
           1.0 / float(tau), _ptr(bonus), float(q_scale), state.data_ptr(), ctx.q_start.data_ptr(), ctx.state_slots.data_ptr(),
-          out.data_ptr(), R, heads, dim, vdim, _code(q.dtype), _stream())
+          out.data_ptr(), R, heads, dim, vdim, RECURRENCE_STRETCH, stretches, _ptr(pair_a), _ptr(pair_b), _code(q.dtype),
+          _stream())
     return out
 
 

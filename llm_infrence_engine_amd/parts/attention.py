@@ -62,11 +62,6 @@ class GQAttention(Mixer):
         self.names = dict(_NAMES, **dict(names or {}))
         self.slopes = self.w_gate_rows = None
 
-    @property
-    def _extras(self) -> bool:
-        """Whether attention needs more than the causal (windowed) softmax with an optional sink."""
-        return bool(self.softcap or self.slope_base is not None or self.gate or self.out_scale != 1.0)
-
     def _bias_name(self, which: str) -> str:
         name = self.names[which]
         if self.bias_suffix is not None:
@@ -97,14 +92,17 @@ class GQAttention(Mixer):
         by_name = {s.name: s for s in GQAttention.tensor_specs(self)}
         p = self.prefix
         w = [get(by_name[p + self.names[n]]) for n in ("q", "k", "v")]
-        if self.gate:       # the gate's rows ride on the packed product, after q, k and v
-            w.append(get(by_name[p + self.names["gate"]]))
+        if self.gate:       # the gate's rows ride on the packed product, after q, k and v; rows of zeros make the
+            w.append(get(by_name[p + self.names["gate"]]))      # product's rows a multiple of 16 bytes, as the matrix-core attention reads q
+            pad = (-sum(t.shape[0] for t in w)) % 8
+            if pad:
+                w.append(torch.zeros(pad, self.hidden_size, dtype=w[0].dtype, device=w[0].device))
         self.w_qkv = linear.prepare_weight(torch.cat(w, dim=0))
         self.b_qkv = None
         if self.qkv_bias:
             b = [get(by_name[p + self._bias_name(n)]) for n in ("q", "k", "v")]
             if self.gate:
-                b.append(torch.zeros(self.num_heads, dtype=b[0].dtype, device=b[0].device))
+                b.append(torch.zeros(self.w_qkv.shape[0] - sum(t.numel() for t in b), dtype=b[0].dtype, device=b[0].device))
             self.b_qkv = torch.cat(b).contiguous()
         self.w_o = linear.prepare_weight(get(by_name[p + self.names["o"]]))
         self.b_o = get(by_name[p + self._bias_name("o")]) if self.out_bias else None
@@ -122,7 +120,7 @@ class GQAttention(Mixer):
     def cache_need(self):
         # in bfloat16 the matrix-core attention reads value pages as an operand as they lie, transposed, which it
         # can for pages of a multiple of 16 tokens
-        if self.value_dim == self.head_dim and not self._extras:
+        if self.value_dim == self.head_dim:
             return KVNeed(self.num_kv_heads, self.head_dim, self.window, transpose_values_at=16,
                           transpose_values_in=torch.bfloat16)
         return CacheNeed((PageTensor("k", self.num_kv_heads, self.head_dim),
@@ -177,7 +175,7 @@ class GQAttention(Mixer):
             self.position.encode_and_store(qkv, nh, nkv, d, ctx, kv)
         out = self.rt.empty(ctx.num_tokens, nh * dv)
         ops.paged_attention(qkv, kv, ctx, out, nh, self.scale, self.window, self.sink_w, self.softcap, self.slopes,
-                            proj[:, width:], self.out_scale)
+                            proj[:, width:width + nh], self.out_scale)
         return linear.linear_residual(out, self.w_o, self.b_o, x)
 
 
