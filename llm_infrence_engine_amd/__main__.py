@@ -19,7 +19,7 @@ def _ids(text: str):
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="python -m llm_infrence_engine_amd", description=__doc__.split("\n\n")[0])
     ap.add_argument("--model", help="folder with config.json and *.safetensors")
-    ap.add_argument("--random-config", help="instead of --model: a preset (tinyA, tinyB, 0.5b, 7b, 32b, gemadra-0.5b, gemadra-7b, gidurax-0.5b, gidurax-7b, kuvazen-0.5b, kuvazen-7b) or the path of a "
+    ap.add_argument("--random-config", help="instead of --model: a preset (tinyA, tinyB, 0.5b, 7b, 32b, gemadra-0.5b, gemadra-7b, gidurax-0.5b, gidurax-7b, kuvazen-0.5b, kuvazen-7b, silizen-0.5b, silizen-7b) or the path of a "
                                             "config.json, filled with random weights drawn on the GPU")
     ap.add_argument("--seed", type=int, default=0, help="seed of the random weights")
     ap.add_argument("--dtype", default="bfloat16", choices=["float32", "bfloat16"])
