@@ -23,7 +23,18 @@ namespace {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_QKV = 2, EPI_GROUPED = 3 };
+enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_QKV = 2, EPI_GROUPED = 3, EPI_GEGLU = 4 };
+
+// the gate's activation of a gated epilogue: g * sigmoid(g), or the tanh form of the gelu with the tanh as
+// 1 - 2 / (2^(2 y log2 e) + 1) through the hardware's exp2 and reciprocal (the result is rounded to bfloat16)
+template <int EPI> __device__ __forceinline__ float gate_act(float g) {
+  if (EPI == EPI_GEGLU) {
+    const float y = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(2.885390081777927f * y) + 1.0f);
+    return 0.5f * g * (1.0f + t);
+  }
+  return fast_silu(g);
+}
 
 // What the grouped product needs beside the operands: the token tiles are tiles of rows that belong to one expert each
 // (ms_moe_align's lists), W holds the experts' matrices one after the other, rows of A are gathered and rows of the
@@ -288,13 +299,13 @@ gemm_tiled_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restrict
   for (int j = 0; j < TT; ++j) {
     const int m = m0 + wt * TT * 16 + j * 16 + col;
     if (m >= M) continue;
-    if (EPI == EPI_SWIGLU) {   // features 2g, 2g + 1 are gate g and up g: 2 FT outputs from o0 on
+    if (EPI == EPI_SWIGLU || EPI == EPI_GEGLU) {   // features 2g, 2g + 1 are gate g and up g: 2 FT outputs from o0 on
       const int o0 = f0 / 2, n_out = N / 2;
       float v[2 * FT];
 #pragma unroll
       for (int i = 0; i < FT; ++i) {
-        v[2 * i] = fast_silu(acc[i][j][0]) * acc[i][j][1];
-        v[2 * i + 1] = fast_silu(acc[i][j][2]) * acc[i][j][3];
+        v[2 * i] = gate_act<EPI>(acc[i][j][0]) * acc[i][j][1];
+        v[2 * i + 1] = gate_act<EPI>(acc[i][j][2]) * acc[i][j][3];
       }
       store_run<2 * FT>(reinterpret_cast<bf16*>(out) + (size_t)m * ldo + o0, v, n_out - o0);
     } else if (EPI == EPI_GROUPED) {
@@ -424,19 +435,22 @@ extern "C" int ms_gemm_tiled_pays(int M, int N, int K) {
 }
 
 // A bfloat16 [M, lda], W bfloat16 [N, ldw] (rows of K, K a multiple of 64), out bfloat16.
-// epilogue 0: out[M, N] = product;  epilogue 1: out[M, N / 2] = silu(gate) * up over interleaved rows of W.
+// epilogue 0: out[M, N] = product;  epilogue 1: out[M, N / 2] = silu(gate) * up over interleaved rows of W;
+// epilogue 4: the same with the tanh form of the gelu for the silu.
 extern "C" int ms_gemm_tiled(const void* A, long long lda, const void* W, long long ldw, void* out, long long ldo, int M,
                              int N, int K, int epilogue, hipStream_t stream) {
   if (M <= 0 || N <= 0) return MS_OK;
   if (K <= 0 || K % BK || lda % 8 || ldw % 8 || lda < K || ldw < K) return MS_UNSUPPORTED;
   if (((uintptr_t)A | (uintptr_t)W) % 16) return MS_UNSUPPORTED;
-  if (epilogue == EPI_SWIGLU ? (N % 2 || ldo < N / 2) : (epilogue != EPI_STORE || ldo < N)) return MS_BAD_ARG;
+  const bool gated = epilogue == EPI_SWIGLU || epilogue == EPI_GEGLU;
+  if (gated ? (N % 2 || ldo < N / 2) : (epilogue != EPI_STORE || ldo < N)) return MS_BAD_ARG;
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
   bf16* o = (bf16*)out;
   int tile = g_tile;
   if (tile == 0) tile = choose_tile(M, N, K).tile;
 #define GO(WF, WT, FT, TT) return epilogue == EPI_SWIGLU ? launch<WF, WT, FT, TT, EPI_SWIGLU, bf16>(a, lda, w, ldw, o, ldo, M, N, K, stream) \
+                                : epilogue == EPI_GEGLU ? launch<WF, WT, FT, TT, EPI_GEGLU, bf16>(a, lda, w, ldw, o, ldo, M, N, K, stream)  \
                                                         : launch<WF, WT, FT, TT, EPI_STORE, bf16>(a, lda, w, ldw, o, ldo, M, N, K, stream)
   if (tile == 1) GO(2, 4, 8, 4);   // 256 x 256
   if (tile == 3) GO(1, 4, 4, 1);   // 64 x 64, four waves

@@ -465,6 +465,7 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Opti
 
 SKINNY_MAX_ROWS = 64
 EPI_STORE, EPI_SWIGLU, EPI_RESIDUAL = 0, 1, 3
+EPI_GEGLU = 4      # as EPI_SWIGLU with the tanh form of the gelu (the tiled product alone has it)
 
 
 def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
@@ -536,14 +537,14 @@ def gemm_tiled_plain_pays(a: torch.Tensor, w: torch.Tensor) -> bool:
 def gemm_tiled(a: torch.Tensor, w: torch.Tensor, epilogue: int = EPI_STORE) -> torch.Tensor:
     """a [M, K] @ w [N, K].T for many rows on the matrix cores, bfloat16 in and out: EPI_STORE -> [M, N];
     EPI_SWIGLU over interleaved rows of w (2j: gate j, 2j + 1: up j) -> [M, N / 2], the product itself never
-    written.  K a multiple of 64 (else ``UnsupportedShape``)."""
+    written; EPI_GEGLU: the same with gelu_tanh(gate) for silu(gate).  K a multiple of 64 (else ``UnsupportedShape``)."""
     _check(a, "a", torch.bfloat16)
     _check(w, "w", torch.bfloat16, (None, a.shape[1]))
-    if epilogue not in (EPI_STORE, EPI_SWIGLU):
+    if epilogue not in (EPI_STORE, EPI_SWIGLU, EPI_GEGLU):
         raise ValueError("the tiled product stores its result or the gated activation of it")
     M, K = a.shape
     N = w.shape[0]
-    out = torch.empty((M, N // 2 if epilogue == EPI_SWIGLU else N), dtype=torch.bfloat16, device=a.device)
+    out = torch.empty((M, N // 2 if epilogue in (EPI_SWIGLU, EPI_GEGLU) else N), dtype=torch.bfloat16, device=a.device)
     _call("ms_gemm_tiled", a.data_ptr(), K, w.data_ptr(), K, out.data_ptr(), out.shape[1], M, N, K, epilogue, _stream())
     return out
 

@@ -122,8 +122,15 @@ class GatedGLU(FeedForward):
         if self.activation == "silu":
             act = linear.linear_swiglu(h, self.w_gate_up)
         else:
-            gu = linear.linear(h, self.w_gate_up)
-            act = ops.gelu_tanh_glu(gu, self.rt.empty(gu.shape[0], self.intermediate_size))
+            act = None
+            if h.dtype == torch.bfloat16 and h.shape[0] > ops.SKINNY_MAX_ROWS and ops.gemm_tiled_pays(h, self.w_gate_up):
+                try:        # many rows: the activation is the product's epilogue
+                    act = ops.gemm_tiled(h, self.w_gate_up, ops.EPI_GEGLU)
+                except ops.UnsupportedShape:
+                    act = None
+            if act is None:
+                gu = linear.linear(h, self.w_gate_up)
+                act = ops.gelu_tanh_glu(gu, self.rt.empty(gu.shape[0], self.intermediate_size))
         return linear.linear_residual(act, self.w_down, None, x)
 
 

@@ -653,6 +653,20 @@ def test_small_kernels_between_the_products(dtype):
     assert (got.cpu().double() - want).abs().max() < tol
 
 
+@gpu
+@pytest.mark.parametrize("M,K,F_", [(200, 128, 96), (70, 64, 40), (513, 256, 320)])
+def test_gated_product_with_the_tanh_gelu_as_its_epilogue(M, K, F_):
+    from llm_infrence_engine_amd.kernels import linear, ops
+
+    g = torch.Generator().manual_seed(M)
+    a = torch.randn(M, K, generator=g).bfloat16()
+    gate, up = (torch.randn(F_, K, generator=g) / math.sqrt(K) * 2).bfloat16(), (torch.randn(F_, K, generator=g) / math.sqrt(K)).bfloat16()
+    w = linear.interleave_rows(gate.cuda(), up.cuda())
+    got = ops.gemm_tiled(a.cuda(), w, ops.EPI_GEGLU)
+    want = P.gelu_tanh(a.double() @ gate.double().T) * (a.double() @ up.double().T)
+    assert got.shape == (M, F_) and ((got.cpu().double() - want).abs() / want.abs().clamp(min=1.0)).max() < 2e-2
+
+
 # ================================================================================================ whole models
 def rounded_forward(cfg, w, toks):
     exact = P.forward(cfg, w, toks)
