@@ -87,8 +87,15 @@ SHAPES["S"] = config(257, 160, 1e-5, 0.25, [
 SHAPES["T"] = config(77, 100, 1e-5, 0.8, [
     parallel(rotated(5, 5, 10, 14, 0.3, 8.0, 10000.0, 6), 2, 18, 26, 2.0, 0.9, 1.0, dense(36)),
     parallel_2(2, 2, 14, 10, 0.3, None, 3, 1, 10, 14, 3, None)], loop=(0, 2, 2))
-PAGES = {"P": 16, "Q": 8, "R": 4, "S": 16, "T": 16}
-SEEDS = {"P": 84, "Q": 92, "R": 81, "S": 98, "T": 82}
+# heads of 128 (one key/value head for four query heads), a window of several pages, every entry of a head rotated, wide
+# recurrences, the first layer alone walked three times
+SHAPES["U"] = config(301, 256, 1e-5, 0.3, [
+    parallel_2(4, 1, 128, 128, 0.09, 50, 2, 1, 128, 96, 4, dense(256)),
+    parallel(rotated(4, 2, 128, 128, 0.09, 12.0, 1000000.0, 128, (2.0, 1.0, 8.0, 256)), 2, 128, 64, 16.0, 0.6, 1.1, dense(192)),
+    wkv(2, 128, dense(128))], loop=(0, 1, 3))
+RANKS["U"] = {0: (16, 24), 1: (16,), 2: (32,)}
+PAGES = {"P": 16, "Q": 8, "R": 4, "S": 16, "T": 16, "U": 16}
+SEEDS = {"P": 84, "Q": 92, "R": 81, "S": 98, "T": 82, "U": 77}
 
 
 def tensor_shapes(cfg, ranks):
@@ -680,7 +687,7 @@ def shape(request, tmp_path_factory):
     weights = random_weights(cfg, RANKS[name], seed=SEEDS[name])
     folder = write_model(tmp_path_factory.mktemp("silizen" + name), cfg, weights)
     lengths = {"P": [5, 61, 2, 130, 33, 48], "Q": [1, 9, 90, 47, 110, 64], "R": [3, 26, 70, 17, 2, 41, 60, 33],
-               "S": [70, 3, 140, 50, 97, 33], "T": [40, 2, 90, 17, 66]}[name]
+               "S": [70, 3, 140, 50, 97, 33], "T": [40, 2, 90, 17, 66], "U": [120, 5, 64, 33]}[name]
     reqs = requests_for(cfg["vocab"], lengths, seed=ord(name))
     w64 = {k: v.double() for k, v in weights.items()}
     want, noise = {}, {}
