@@ -186,13 +186,13 @@ class SilizenConfig:
         return total
 
     # ------------------------------------------------------------------ the model as data
-    def _attention(self, p: str, left: dict, kind: str) -> Tuple[PartSpec, PartSpec]:
-        """(mixer PartSpec, position PartSpec) of an attention half."""
+    def _attention(self, p: str, left: dict, kind: str, out_scale: float = 1.0) -> Tuple[PartSpec, PartSpec]:
+        """(mixer PartSpec, position PartSpec) of an attention half; ``out_scale``: the half's weight in the mixer's sum."""
         W, eps = self.width, self.norm_eps
         names = {"q": "q", "k": "k", "v": "v", "o": "o", "gate": "g"}
         common = {"hidden_size": W, "num_heads": left["heads"], "num_kv_heads": left["kv_heads"], "head_dim": left["dim"],
                   "value_dim": left["vdim"], "scale": float(left["scale"]), "out_bias": False, "sink": "zero", "gate": True,
-                  "names": names, "bias_suffix": ".b"}
+                  "names": names, "bias_suffix": ".b", "out_scale": float(out_scale)}
         if kind == "parallel":
             rot = left.get("rot") or {}
             position = PartSpec("qk_norm_rotary_half", p, {
@@ -211,15 +211,17 @@ class SilizenConfig:
         if kind == "wkv":
             return PartSpec("wkv", p, {"hidden_size": W, "heads": m["heads"], "dim": m["dim"], "eps": eps,
                                        "decay_rank": self._rank(i, entry, "decay_rank")})
-        left, left_position = self._attention(p + "left.", m["left"], kind)
         r = m["right"]
         if kind == "parallel":
+            # the halves' weights ride on kernels that are there anyway (the attention's normalisation, the read-out's norm),
+            # so that each half's output product can add straight into the residual stream
+            left, left_position = self._attention(p + "left.", m["left"], kind, out_scale=float(m["left_scale"]))
             right = PartSpec("gated_linear_attention", p + "right.", {
                 "hidden_size": W, "heads": r["heads"], "dim": r["dim"], "vdim": r["vdim"], "tau": float(r["tau"]), "eps": eps,
-                "decay_rank": self._rank(i, entry, "right.decay_rank")})
+                "decay_rank": self._rank(i, entry, "right.decay_rank"), "out_scale": float(m["right_scale"])})
             return PartSpec("side_by_side", p, {"hidden_size": W, "left": left, "right": right, "left_position": left_position,
-                                                "combine": "scaled", "left_scale": float(m["left_scale"]),
-                                                "right_scale": float(m["right_scale"])})
+                                                "combine": "scaled"})
+        left, left_position = self._attention(p + "left.", m["left"], kind)
         right = PartSpec("gated_delta", p + "right.", {
             "hidden_size": W, "heads": r["heads"], "kv_heads": r["kv_heads"], "dim": r["dim"], "vdim": r["vdim"],
             "taps": r["conv"], "eps": eps, "decay": "channel", "gate": "low_rank_sigmoid",

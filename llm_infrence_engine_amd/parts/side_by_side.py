@@ -1,6 +1,8 @@
 """Two mixers side by side: both read the same input h, and the layer's mixer result is a sum of the two.
 
-``combine`` = "scaled": left_scale * left(h) + right_scale * right(h).
+``combine`` = "scaled": left_scale * left(h) + right_scale * right(h).  With both scales one (a configuration may hand the
+scales to the halves themselves, where they ride on a kernel that is there anyway) every half adds its result into the
+residual stream through its own last product, and only what a half hands back is summed here.
 ``combine`` = "normed_mean": (RMS(left(h)) o w_left + RMS(right(h)) o w_right) / 2, each result divided by its root mean
 square over the model's width (eps inside the root) and multiplied by a stored weight of its own (``left_norm_name`` /
 ``right_norm_name`` after the prefix).
@@ -93,6 +95,18 @@ class SideBySide(Mixer):
         return x
 
     def forward_residual(self, h, ctx, kv, state, x):
+        if self.combine == "scaled" and self.left_scale == 1.0 and self.right_scale == 1.0:
+            handed = []
+            for i, m in enumerate(self.halves):
+                mine = kv if m.cache_need() is not None else None
+                r = m.forward_residual(h, ctx, mine, self._state_of(i, state), x)
+                if r is not None:
+                    handed.append(r)
+            if len(handed) == 2:
+                ops.pair_sum(x, handed[0], handed[1])
+            elif handed:
+                ops.residual_add(x, handed[0])
+            return None
         results = []
         for i, m in enumerate(self.halves):
             mine = kv if m.cache_need() is not None else None
